@@ -27,7 +27,7 @@ from typing import Hashable
 import numpy as np
 import torch
 
-from ..parts.base import CompositeSpec, FixedStateSpec, LayerCache, PagedSpec, paged_specs
+from ..parts.base import BorrowedCache, CompositeSpec, FixedStateSpec, LayerCache, PagedSpec, paged_specs
 from .pool import CacheError, OutOfPages, PagePool
 
 RELEASED = -1     # host-side mark of a logical page a window has passed
@@ -75,25 +75,47 @@ class CacheManager:
         self.layer_caches: list[LayerCache | None] = [None] * len(needs)
         self._by_need: dict[tuple[int | None, int, int], int] = {}
         self._allocate = bool(allocate_tensors)
+        self._borrowed: list[tuple[LayerCache, str, BorrowedCache, int]] = []
         for run, need in enumerate(needs):
             if isinstance(need, (PagedSpec, FixedStateSpec, CompositeSpec)):
                 self.layer_caches[run] = self._build(need, run)
         for run, need in enumerate(needs):          # runs that read an earlier run's cache
             if isinstance(need, int) and not isinstance(need, bool):
-                source = self.layer_caches[need]
-                if source is None:
-                    raise CacheError(f"run {run} reads the cache of run {need}, which has none")
-                self.layer_caches[run] = LayerCache(source.spec, source.group, tensors=source.tensors,
-                                                    state=source.state, writes=False, page_size=source.page_size,
-                                                    children=source.children)
+                self.layer_caches[run] = self._reader(self._lent(BorrowedCache(need), run))
+        for holder, name, borrowed, run in self._borrowed:      # parts of a composite that read an earlier run's
+            holder.children[name] = self._reader(self._lent(borrowed, run))
         self._requests: dict[Hashable, RequestCache] = {}
         self._free_slots = list(range(self.max_requests - 1, -1, -1))
         self.padding_state_slot = self.max_requests       # never handed to a request
 
+    def _lent(self, borrowed: BorrowedCache, run: int) -> LayerCache:
+        """The cache (or the named part of it) of the earlier run that ``run`` reads."""
+        if not 0 <= borrowed.run < run:
+            raise CacheError(f"run {run} reads the cache of run {borrowed.run}: only an earlier run's can be read")
+        source = self.layer_caches[borrowed.run]
+        for name in borrowed.path:
+            source = source.children.get(name) if source is not None else None
+        if source is None:
+            where = f"run {borrowed.run}" + "".join(f".{name}" for name in borrowed.path)
+            raise CacheError(f"run {run} reads the cache of {where}, which has none")
+        return source
+
+    @staticmethod
+    def _reader(source: LayerCache) -> LayerCache:
+        return LayerCache(source.spec, source.group, tensors=source.tensors, state=source.state, writes=False,
+                          page_size=source.page_size,
+                          children={name: CacheManager._reader(child) for name, child in source.children.items()})
+
     def _build(self, need: "PagedSpec | FixedStateSpec | CompositeSpec", run: int) -> LayerCache:
         """The cache of one run (or of one part of a run whose mixer is made of several)."""
         if isinstance(need, CompositeSpec):
-            return LayerCache(need, -1, children={name: self._build(part, run) for name, part in need.parts})
+            holder = LayerCache(need, -1)
+            for name, part in need.parts:
+                if isinstance(part, BorrowedCache):
+                    self._borrowed.append((holder, name, part, run))      # resolved once every run is built
+                else:
+                    holder.children[name] = self._build(part, run)
+            return holder
         if isinstance(need, PagedSpec):
             page_size = int(need.page_size or self.block_size)
             keep_first = int(need.keep_first) if need.window is not None else 0
@@ -121,7 +143,7 @@ class CacheManager:
     def state_caches(self) -> list[LayerCache]:
         """Every cache that holds per-request state of fixed size and is written by its run."""
         return [leaf for cache in self.layer_caches if cache is not None and cache.writes
-                for leaf in cache.leaves() if leaf.state is not None]
+                for leaf in cache.leaves() if leaf.state is not None and leaf.writes]
 
     @property
     def pool_tokens(self) -> int:

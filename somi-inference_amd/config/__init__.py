@@ -4,6 +4,8 @@ from .base import ConfigError, KeyReader, ModelConfig, architecture_of, read_con
 from .engine import (DEFAULT_BLOCK_SIZE, DEFAULT_MAX_CONCURRENT, DEFAULT_NUM_BLOCKS,
                      EngineConfig, normalize_dtype)
 from .kamedra import KamedraAttention, KamedraConfig, KamedraGLA, KamedraLayer, RotaryScaling
+from .metitar import (MetitarConfig, MetitarDense, MetitarExperts, MetitarHGRN2, MetitarLatentAttention, MetitarLayer,
+                      RampedScaling)
 from .qwen2 import Qwen2Config
 from .rusolorn import RusolornAttention, RusolornConfig, RusolornDeltaRule, RusolornExperts, RusolornLayer
 from .registry import (Architecture, config_from_dict, register_architecture,
@@ -12,6 +14,7 @@ from .registry import (Architecture, config_from_dict, register_architecture,
 __all__ = [
     "Architecture", "ConfigError", "DEFAULT_BLOCK_SIZE", "DEFAULT_MAX_CONCURRENT",
     "DEFAULT_NUM_BLOCKS", "EngineConfig", "KamedraAttention", "KamedraConfig", "KamedraGLA", "KamedraLayer", "KeyReader",
+    "MetitarConfig", "MetitarDense", "MetitarExperts", "MetitarHGRN2", "MetitarLatentAttention", "MetitarLayer", "RampedScaling",
     "ModelConfig", "Qwen2Config", "RotaryScaling", "RusolornAttention", "RusolornConfig", "RusolornDeltaRule",
     "RusolornExperts", "RusolornLayer",
     "architecture_of", "config_from_dict", "normalize_dtype", "read_config_json",

@@ -129,3 +129,48 @@ extern "C" int somi_softcap(float* x, float cap, int64_t count, hipStream_t stre
     SOMI_LAUNCH_CHECK("softcap");
     return 0;
 }
+
+// A polynomial activation with normed powers: for a row z of float32 sums,
+//
+//     out = a N(z) + b N(z^2) + c N(z^3) + e,     N(u) = u / sqrt(mean(u^2) + eps) over the row,
+//
+// powers element by element; coef = (a, b, c, e) on the device.  One workgroup per row; the three mean squares are
+// float32, the result is rounded once.
+template <typename TO>
+__global__ void __launch_bounds__(256)
+poly_norm_kernel(const float* __restrict__ z, const float* __restrict__ coef, float eps, TO* __restrict__ out, int width) {
+    __shared__ float red[16];
+    const float* row = z + (int64_t)blockIdx.x * width;
+    float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    for (int i = threadIdx.x; i < width; i += 256) {
+        const float v = row[i], v2 = v * v, v3 = v2 * v;
+        s1 = fmaf(v, v, s1);
+        s2 = fmaf(v2, v2, s2);
+        s3 = fmaf(v3, v3, s3);
+    }
+    s1 = block_sum<256>(s1, red);
+    s2 = block_sum<256>(s2, red);
+    s3 = block_sum<256>(s3, red);
+    const float n = (float)width;
+    const float r1 = coef[0] / sqrtf(s1 / n + eps), r2 = coef[1] / sqrtf(s2 / n + eps), r3 = coef[2] / sqrtf(s3 / n + eps);
+    const float shift = coef[3];
+    TO* o = out + (int64_t)blockIdx.x * width;
+    for (int i = threadIdx.x; i < width; i += 256) {
+        const float v = row[i], v2 = v * v;
+        o[i] = from_float<TO>(r1 * v + r2 * v2 + r3 * (v2 * v) + shift);
+    }
+}
+
+extern "C" int somi_poly_norm(const float* z, const float* coef, float eps, void* out, int out_dtype, int n_tokens, int width,
+                              hipStream_t stream) {
+    SOMI_REQUIRE(n_tokens >= 0 && width > 0, "poly_norm: bad sizes");
+    if (n_tokens == 0) return 0;
+    if (out_dtype == SOMI_F32)
+        hipLaunchKernelGGL(poly_norm_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, z, coef, eps, (float*)out, width);
+    else if (out_dtype == SOMI_BF16)
+        hipLaunchKernelGGL(poly_norm_kernel<bf16>, dim3(n_tokens), dim3(256), 0, stream, z, coef, eps, (bf16*)out, width);
+    else
+        return somi_fail("poly_norm: unknown dtype %d", out_dtype);
+    SOMI_LAUNCH_CHECK("poly_norm");
+    return 0;
+}

@@ -251,8 +251,9 @@ extern "C" int somi_gla_scan(const void* q, const void* k, const void* v, int dt
 }
 
 // ------------------------------------------------------------------------------------------------ norm and gate
-// y[t, h, c] = o / sqrt(mean_c(o^2) + eps) * w[c] * silu(g[t, h, c]).  One wavefront per (token, head).
-template <typename T>
+// y[t, h, c] = o / sqrt(mean_c(o^2) + eps) * w[c] * silu(g[t, h, c]); without a gate (GATE false) the last factor is
+// left out.  One wavefront per (token, head).
+template <typename T, bool GATE>
 __global__ void __launch_bounds__(64)
 gla_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w, const T* __restrict__ g,
                      int64_t g_stride, float eps, T* __restrict__ y, int heads, int vdim) {
@@ -263,8 +264,12 @@ gla_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w, c
     for (int c = lane; c < vdim; c += 64) ss = fmaf(orow[c], orow[c], ss);
     ss = wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
-    const T* grow = g + t * g_stride + (int64_t)h * vdim;
     T* yrow = y + (t * heads + h) * vdim;
+    if (!GATE) {
+        for (int c = lane; c < vdim; c += 64) yrow[c] = from_float<T>(orow[c] * inv * w[c]);
+        return;
+    }
+    const T* grow = g + t * g_stride + (int64_t)h * vdim;
     for (int c = lane; c < vdim; c += 64) {
         const float gate = to_float(grow[c]);
         const float silu = gate / (1.0f + expf(-gate));
@@ -272,22 +277,63 @@ gla_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w, c
     }
 }
 
-// o: [n_tokens, heads, vdim] float32; w: [vdim] float32; g: [n_tokens, g_stride] with head h at h * vdim ..;
-// y: [n_tokens, heads * vdim] in the storage type.
+// o: [n_tokens, heads, vdim] float32; w: [vdim] float32; g: [n_tokens, g_stride] with head h at h * vdim .., or null
+// for a mixer without a gate; y: [n_tokens, heads * vdim] in the storage type.
 extern "C" int somi_gla_norm_gate(const float* o, const float* w, const void* g, int dtype, int64_t g_stride, float eps,
                                   void* y, int n_tokens, int heads, int vdim, hipStream_t stream) {
-    SOMI_REQUIRE(n_tokens >= 0 && heads > 0 && vdim > 0 && g_stride >= (int64_t)heads * vdim, "gla_norm_gate: bad sizes");
+    SOMI_REQUIRE(n_tokens >= 0 && heads > 0 && vdim > 0 && (g == nullptr || g_stride >= (int64_t)heads * vdim),
+                 "gla_norm_gate: bad sizes");
     SOMI_REQUIRE(heads <= 65535, "gla_norm_gate: too many heads");
     if (n_tokens == 0) return 0;
     const dim3 grid(n_tokens, heads);
-    if (dtype == SOMI_F32)
-        hipLaunchKernelGGL(gla_norm_gate_kernel<float>, grid, dim3(64), 0, stream, o, w, (const float*)g, g_stride, eps,
-                           (float*)y, heads, vdim);
-    else if (dtype == SOMI_BF16)
-        hipLaunchKernelGGL(gla_norm_gate_kernel<bf16>, grid, dim3(64), 0, stream, o, w, (const bf16*)g, g_stride, eps,
-                           (bf16*)y, heads, vdim);
-    else
+#define GLA_NORM(T, GATE)                                                                                            \
+    hipLaunchKernelGGL((gla_norm_gate_kernel<T, GATE>), grid, dim3(64), 0, stream, o, w, (const T*)g, g_stride, eps, \
+                       (T*)y, heads, vdim)
+    if (dtype == SOMI_F32) {
+        if (g) GLA_NORM(float, true); else GLA_NORM(float, false);
+    } else if (dtype == SOMI_BF16) {
+        if (g) GLA_NORM(bf16, true); else GLA_NORM(bf16, false);
+    } else {
         return somi_fail("gla_norm_gate: unknown dtype %d", dtype);
+    }
+#undef GLA_NORM
     SOMI_LAUNCH_CHECK("gla_norm_gate");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------ bounded forget gates
+// For a recurrence whose forget gate also decides what is written (S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T, o_t =
+// S_t^T q_t): from rows [q as projected | z, the gate's projection | ...] of float32 sums, in place,
+//
+//     q <- silu(q);     f = lower + (1 - lower) sigmoid(z + bias);     z <- 1 - f = (1 - lower) sigmoid(-(z + bias))
+//
+// and f itself into `decay`, so that the recurrence above reads q, k = 1 - f and alpha = f.  lower, bias: [width], the
+// heads' channels in one row.
+__global__ void __launch_bounds__(256)
+bounded_forget_kernel(float* __restrict__ rows, int64_t row_stride, const float* __restrict__ bias,
+                      const float* __restrict__ lower, float* __restrict__ decay, int width, int64_t count) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t)gridDim.x * 256) {
+        const int64_t t = i / width;
+        const int c = (int)(i - t * width);
+        float* row = rows + t * row_stride;
+        const float q = row[c];
+        row[c] = q / (1.0f + expf(-q));
+        const float z = row[width + c] + bias[c];
+        const float lo = lower[c];
+        const float keep = 1.0f / (1.0f + expf(-z)), write = 1.0f / (1.0f + expf(z));
+        decay[i] = lo + (1.0f - lo) * keep;
+        row[width + c] = (1.0f - lo) * write;
+    }
+}
+
+extern "C" int somi_bounded_forget(float* rows, int64_t row_stride, const float* bias, const float* lower, float* decay,
+                                   int n_tokens, int width, hipStream_t stream) {
+    SOMI_REQUIRE(n_tokens >= 0 && width > 0 && row_stride >= 2 * (int64_t)width, "bounded_forget: bad sizes");
+    const int64_t count = (int64_t)n_tokens * width;
+    if (count == 0) return 0;
+    const int grid = (int)(ceil_div64(count, 256) < 65536 ? ceil_div64(count, 256) : 65536);
+    hipLaunchKernelGGL(bounded_forget_kernel, dim3(grid), dim3(256), 0, stream, rows, row_stride, bias, lower, decay, width,
+                       count);
+    SOMI_LAUNCH_CHECK("bounded_forget");
     return 0;
 }

@@ -1,13 +1,16 @@
 // Mixture of experts: the router, the grouping of (token, expert) pairs by expert, the experts' products over the
 // grouped rows and the weighted sum.
 //
-//   route      z = W_r h (float32), s = softmax(z); experts come in `groups` equal runs of neighbours, a run scores as
-//              its best expert and only the `keep` best runs stay; of their experts the `top` with the largest s are
-//              chosen, weighted by s over the chosen scores' sum (+ 1e-20).  Ties go to the lower index.
+//   route      z = W_r h (float32), s = softmax(z) or, element by element, sigmoid(z); experts come in `groups` equal
+//              runs of neighbours, a run scores as its best expert and only the `keep` best runs stay; of their experts
+//              the `top` with the largest s are chosen, weighted by s over the chosen scores' sum (+ 1e-20) or by s as
+//              it is.  Ties go to the lower index.
 //   align      the N * top pairs sorted by expert: order[], the experts' offsets and a list of row tiles
 //              (expert, first sorted row, rows) that the products' grids walk.
-//   gate_up    act[p, :] = glu(W_gate[e] h_t, W_up[e] h_t) for the sorted pair p = (t, e)
-//   down       y[pair, :] = w_pair * (W_down[e] act[p, :]), float32, at the pair's own place t * top + j
+//   gate_up    act[p, :] = glu(W_gate[e] h_t, W_up[e] h_t) for the sorted pair p = (t, e); where the pair's weight is to
+//              multiply the expert's input, glu(w_pair W_gate[e] h_t, w_pair W_up[e] h_t): the float32 sums are scaled
+//   down       y[pair, :] = w_pair * (W_down[e] act[p, :]) (or without the weight), float32, at the pair's own place
+//              t * top + j
 //   combine    out[t, :] = sum_j y[t * top + j, :] (+ shared[t, :]), float32, in the order of j
 //
 // glu(g, u) = g' sigmoid(alpha g') (u' + shift) with g' = min(g, limit) and u' = clamp(u, -limit, limit).
@@ -125,7 +128,8 @@ template <typename T>
 __global__ void __launch_bounds__(64)
 moe_route_kernel(const T* __restrict__ x, int64_t row_stride, const float* __restrict__ router,
                  const float* __restrict__ logits, int width, int experts,
-                 int top, int groups, int keep, int* __restrict__ chosen, float* __restrict__ weight) {
+                 int top, int groups, int keep, int sigmoid_scores, int normalize, int* __restrict__ chosen,
+                 float* __restrict__ weight) {
     constexpr int PER_LANE = MOE_MAX_EXPERTS / 64;
     __shared__ float score[MOE_MAX_EXPERTS];
     __shared__ int taken[MOE_MAX_EXPERTS];          // per run: kept or not
@@ -158,10 +162,11 @@ moe_route_kernel(const T* __restrict__ x, int64_t row_stride, const float* __res
     float total = 0.f;
 #pragma unroll
     for (int j = 0; j < PER_LANE; ++j) {
-        s[j] = lane + 64 * j < experts ? expf(s[j] - top_z) : 0.f;
+        if (sigmoid_scores) s[j] = lane + 64 * j < experts ? 1.0f / (1.0f + expf(-s[j])) : 0.f;
+        else s[j] = lane + 64 * j < experts ? expf(s[j] - top_z) : 0.f;
         total += s[j];
     }
-    total = wave_sum(total);
+    total = sigmoid_scores ? 1.0f : wave_sum(total);
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < PER_LANE; ++j) {
@@ -235,13 +240,13 @@ moe_route_kernel(const T* __restrict__ x, int64_t row_stride, const float* __res
     __syncthreads();
     for (int pick = lane; pick < top; pick += 64) {
         chosen[t * top + pick] = pick_index[pick];
-        weight[t * top + pick] = pick_score[pick] / (sum + 1e-20f);
+        weight[t * top + pick] = normalize ? pick_score[pick] / (sum + 1e-20f) : pick_score[pick];
     }
 }
 
 extern "C" int somi_moe_route(const void* x, int dtype, int64_t row_stride, const float* router, float* logits,
-                              int n_tokens, int width, int experts, int top, int groups, int keep, int* chosen,
-                              float* weight, hipStream_t stream) {
+                              int n_tokens, int width, int experts, int top, int groups, int keep, int sigmoid_scores,
+                              int normalize, int* chosen, float* weight, hipStream_t stream) {
     SOMI_REQUIRE(n_tokens >= 0 && width > 0 && experts > 0 && experts <= MOE_MAX_EXPERTS, "moe_route: %d experts, 1 to %d are supported",
                  experts, MOE_MAX_EXPERTS);
     SOMI_REQUIRE(groups >= 1 && experts % groups == 0 && keep >= 1 && keep <= groups, "moe_route: %d groups (keep %d) do not divide %d experts",
@@ -267,10 +272,10 @@ extern "C" int somi_moe_route(const void* x, int dtype, int64_t row_stride, cons
     }
     if (dtype == SOMI_F32)
         hipLaunchKernelGGL(moe_route_kernel<float>, dim3(n_tokens), dim3(64), 0, stream, (const float*)x, row_stride, router,
-                           tiled ? logits : nullptr, width, experts, top, groups, keep, chosen, weight);
+                           tiled ? logits : nullptr, width, experts, top, groups, keep, sigmoid_scores, normalize, chosen, weight);
     else
         hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3(n_tokens), dim3(64), 0, stream, (const bf16*)x, row_stride, router,
-                           tiled ? logits : nullptr, width, experts, top, groups, keep, chosen, weight);
+                           tiled ? logits : nullptr, width, experts, top, groups, keep, sigmoid_scores, normalize, chosen, weight);
     SOMI_LAUNCH_CHECK("moe_route");
     return 0;
 }
@@ -381,11 +386,12 @@ moe_product_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restric
     for (int j = 0; j < 4; ++j) {
         const int c = col0 + cg * 4 + j;
         if (c >= n_out) continue;
+        const int pair = pair_of[r];
+        const float pw = pair_weight != nullptr ? pair_weight[pair] : 1.0f;
         if (GATED) {
-            ((T*)out_)[(int64_t)(first + r) * n_out + c] = from_float<T>(clamped_glu(acc[j], acu[j], limit, alpha, shift));
+            ((T*)out_)[(int64_t)(first + r) * n_out + c] = from_float<T>(clamped_glu(pw * acc[j], pw * acu[j], limit, alpha, shift));
         } else {
-            const int pair = pair_of[r];
-            ((float*)out_)[(int64_t)pair * n_out + c] = pair_weight[pair] * acc[j];
+            ((float*)out_)[(int64_t)pair * n_out + c] = pw * acc[j];
         }
     }
 }
@@ -507,17 +513,17 @@ moe_product_mfma_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16
         for (int i = 0; i < 4; ++i) {
             const int row = f * 16 + g * 4 + i;
             if (row >= rows) continue;
+            const int pair = order[first + row];
+            const float pw = pair_weight != nullptr ? pair_weight[pair] : 1.0f;
             if (GATED) {
 #pragma unroll
                 for (int c = 0; c < 2; ++c) {
                     const int col = col0 + c * 16 + r;
                     if (col < n_out)
                         ((bf16*)out_)[(int64_t)(first + row) * n_out + col] =
-                            (bf16)clamped_glu(acc[f][c][i], acc[f][c + 2][i], limit, alpha, shift);
+                            (bf16)clamped_glu(pw * acc[f][c][i], pw * acc[f][c + 2][i], limit, alpha, shift);
                 }
             } else {
-                const int pair = order[first + row];
-                const float pw = pair_weight[pair];
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     const int col = col0 + c * 16 + r;
@@ -638,14 +644,14 @@ moe_product_tile_kernel(const bf16* __restrict__ a, int64_t a_stride, const bf16
             for (int e = 0; e < 4; ++e) {
                 const int row = wm * 64 + i * 32 + 8 * g + 4 * fk + e;
                 if (row >= rows) continue;
+                const int pair = order[first + row];
+                const float pw = pair_weight != nullptr ? pair_weight[pair] : 1.0f;
                 if (GATED) {
                     const int col = col_base + wn * 32 + frow;
                     if (col < n_out)
                         ((bf16*)out_)[(int64_t)(first + row) * n_out + col] =
-                            (bf16)clamped_glu(acc[i][0][4 * g + e], acc[i][1][4 * g + e], limit, alpha, shift);
+                            (bf16)clamped_glu(pw * acc[i][0][4 * g + e], pw * acc[i][1][4 * g + e], limit, alpha, shift);
                 } else {
-                    const int pair = order[first + row];
-                    const float pw = pair_weight[pair];
 #pragma unroll
                     for (int j = 0; j < 2; ++j) {
                         const int col = col_base + wn * 64 + j * 32 + frow;

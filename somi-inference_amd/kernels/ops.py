@@ -849,12 +849,21 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, alpha: torch.Ten
     return o
 
 
-def gla_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, eps: float) -> torch.Tensor:
+def gla_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor | None, eps: float,
+                  out_dtype: torch.dtype | None = None) -> torch.Tensor:
     """o / sqrt(mean(o^2) + eps) * weight * silu(gate) per head -> [N, heads * vdim] in the gate's dtype.  o: [N, heads,
-    vdim] float32; weight: [vdim] float32; gate: [N, heads * vdim] (a view with a row stride of its own is fine)."""
+    vdim] float32; weight: [vdim] float32; gate: [N, heads * vdim] (a view with a row stride of its own is fine), or None
+    for a mixer without a gate (the result is then in ``out_dtype``)."""
     _need(o, "recurrence output", torch.float32)
     n, heads, vdim = o.shape
     _need(weight, "norm weight", torch.float32, (vdim,))
+    if gate is None:
+        if out_dtype is None:
+            raise KernelError("gla_norm_gate: without a gate the result's dtype must be named")
+        y = torch.empty((n, heads * vdim), dtype=out_dtype, device=o.device)
+        _check(library().somi_gla_norm_gate(_ptr(o), _ptr(weight), None, dtype_code(out_dtype), ctypes.c_int64(0),
+                                            ctypes.c_float(eps), _ptr(y), n, heads, vdim, _stream()))
+        return y
     if (not isinstance(gate, torch.Tensor) or not gate.is_cuda or gate.dim() != 2 or gate.stride(1) != 1
             or tuple(gate.shape) != (n, heads * vdim)):
         raise KernelError(f"gla_norm_gate: the gate must be [{n}, {heads * vdim}] on the GPU with contiguous rows")
@@ -863,6 +872,21 @@ def gla_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, eps
                                         ctypes.c_int64(gate.stride(0)), ctypes.c_float(eps), _ptr(y), n, heads, vdim,
                                         _stream()))
     return y
+
+
+def bounded_forget_(rows: torch.Tensor, width: int, bias: torch.Tensor, lower: torch.Tensor) -> torch.Tensor:
+    """For a recurrence whose forget gate also decides what is written: rows [N, q (width) | z (width) | ...] of float32
+    sums, in place q <- silu(q) and z <- 1 - f with f = lower + (1 - lower) sigmoid(z + bias); returns f [N, width]."""
+    _need(rows, "projected rows", torch.float32)
+    n = rows.shape[0]
+    if rows.dim() != 2 or rows.shape[1] < 2 * width:
+        raise KernelError(f"bounded_forget: rows of {tuple(rows.shape)} do not hold two runs of {width} channels")
+    _need(bias, "gate bias", torch.float32, (width,))
+    _need(lower, "lower bounds", torch.float32, (width,))
+    decay = torch.empty((n, width), dtype=torch.float32, device=rows.device)
+    _check(library().somi_bounded_forget(_ptr(rows), ctypes.c_int64(rows.stride(0)), _ptr(bias), _ptr(lower), _ptr(decay), n,
+                                         int(width), _stream()))
+    return decay
 
 
 def diff_attention_mfma_supported(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor) -> bool:
@@ -1108,20 +1132,27 @@ def moe_mfma_supported(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tenso
             and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and gate_up.data_ptr() % 16 == 0 and down.data_ptr() % 16 == 0)
 
 
-def moe_route(x: torch.Tensor, router: torch.Tensor, top: int, groups: int, keep: int) -> tuple[torch.Tensor, torch.Tensor]:
-    """Chosen experts [N, top] int32 and their weights [N, top] float32 (softmax scores in float32, the ``keep`` best of
-    ``groups`` runs of neighbouring experts, the ``top`` best experts of those, weights over their sum)."""
+ROUTER_SCORES = {"softmax": 0, "sigmoid": 1}
+
+
+def moe_route(x: torch.Tensor, router: torch.Tensor, top: int, groups: int, keep: int, scores: str = "softmax",
+              normalize: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
+    """Chosen experts [N, top] int32 and their weights [N, top] float32: float32 scores (``scores``: the softmax over all
+    experts, or each expert's own sigmoid), the ``keep`` best of ``groups`` runs of neighbouring experts, the ``top`` best
+    experts of those; weights over their sum (``normalize``) or the scores as they are."""
     _need(x, "rows")
     n, width = x.shape
     _need(router, "router", torch.float32)
     if router.dim() != 2 or router.shape[1] != width:
         raise KernelError(f"moe_route: router {tuple(router.shape)} does not fit rows of {width}")
+    if scores not in ROUTER_SCORES:
+        raise KernelError(f"moe_route: unknown scores {scores!r}; known: {sorted(ROUTER_SCORES)}")
     chosen = torch.empty((n, top), dtype=torch.int32, device=x.device)
     weight = torch.empty((n, top), dtype=torch.float32, device=x.device)
     logits = torch.empty((n, router.shape[0]), dtype=torch.float32, device=x.device)     # the router's sums, if it tiles them
     _check(library().somi_moe_route(_ptr(x), dtype_code(x.dtype), ctypes.c_int64(x.stride(0)), _ptr(router), _ptr(logits), n,
-                                    width, router.shape[0], int(top), int(groups), int(keep), _ptr(chosen), _ptr(weight),
-                                    _stream()))
+                                    width, router.shape[0], int(top), int(groups), int(keep), ROUTER_SCORES[scores],
+                                    1 if normalize else 0, _ptr(chosen), _ptr(weight), _stream()))
     return chosen, weight
 
 
@@ -1140,36 +1171,44 @@ def moe_align(chosen: torch.Tensor, experts: int, tile_rows: int = MOE_TILE_ROWS
 
 
 def moe_gate_up(x: torch.Tensor, gate_up: torch.Tensor, tiles: torch.Tensor, order: torch.Tensor, top: int,
-                limit: float, alpha: float, shift: float, tile_rows: int = MOE_TILE_ROWS, mfma: bool = False) -> torch.Tensor:
+                limit: float, alpha: float, shift: float, tile_rows: int = MOE_TILE_ROWS, mfma: bool = False,
+                input_weight: torch.Tensor | None = None) -> torch.Tensor:
     """act[p] = glu(W_gate[e] x[t], W_up[e] x[t]) for the sorted pairs p = (t, e); gate_up: [experts, 2 F, K], gate rows
-    first -> [pairs, F]."""
+    first -> [pairs, F].  ``input_weight`` [pairs] float32: the pair's weight multiplies the expert's input (both float32
+    sums are scaled by it before the unit)."""
     _need(x, "rows")
     _need(gate_up, "gate/up matrices", x.dtype)
     experts, two_f, k = gate_up.shape
     if x.shape[1] != k or two_f % 2:
         raise KernelError(f"moe_gate_up: matrices {tuple(gate_up.shape)} do not fit rows of {x.shape[1]}")
     pairs = order.numel()
+    if input_weight is not None:
+        _need(input_weight, "pair weights", torch.float32)
+        if input_weight.numel() != pairs:
+            raise KernelError(f"moe_gate_up: {input_weight.numel()} weights for {pairs} pairs")
     act = torch.empty((pairs, two_f // 2), dtype=x.dtype, device=x.device)
     if mfma:
         _check(library().somi_moe_product_mfma(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(gate_up), 1, _ptr(tiles), tiles.shape[0],
-                                               int(tile_rows), _ptr(order), None, int(top), two_f // 2, k, ctypes.c_float(limit),
+                                               int(tile_rows), _ptr(order), _ptr(input_weight), int(top), two_f // 2, k, ctypes.c_float(limit),
                                                ctypes.c_float(alpha), ctypes.c_float(shift), _ptr(act), _stream()))
         return act
     _check(library().somi_moe_product(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(gate_up), dtype_code(x.dtype), 1, _ptr(tiles),
-                                      tiles.shape[0], _ptr(order), None, int(top), two_f // 2, k, ctypes.c_float(limit),
+                                      tiles.shape[0], _ptr(order), _ptr(input_weight), int(top), two_f // 2, k, ctypes.c_float(limit),
                                       ctypes.c_float(alpha), ctypes.c_float(shift), _ptr(act), _stream()))
     return act
 
 
-def moe_down(act: torch.Tensor, down: torch.Tensor, tiles: torch.Tensor, order: torch.Tensor, weight: torch.Tensor,
+def moe_down(act: torch.Tensor, down: torch.Tensor, tiles: torch.Tensor, order: torch.Tensor, weight: torch.Tensor | None,
              top: int, tile_rows: int = MOE_TILE_ROWS, mfma: bool = False) -> torch.Tensor:
-    """y[pair] = weight[pair] * W_down[e] act[p] -> [pairs, width] float32, at the pairs' own places."""
+    """y[pair] = weight[pair] * W_down[e] act[p] -> [pairs, width] float32, at the pairs' own places (``weight`` None: the
+    products as they are)."""
     _need(act, "activations")
     _need(down, "down matrices", act.dtype)
     experts, width, k = down.shape
     if act.shape[1] != k:
         raise KernelError(f"moe_down: matrices {tuple(down.shape)} do not fit activations of {act.shape[1]}")
-    _need(weight, "pair weights", torch.float32)
+    if weight is not None:
+        _need(weight, "pair weights", torch.float32)
     y = torch.empty((order.numel(), width), dtype=torch.float32, device=act.device)
     if mfma:
         _check(library().somi_moe_product_mfma(_ptr(act), ctypes.c_int64(act.stride(0)), _ptr(down), 0, _ptr(tiles), tiles.shape[0],
@@ -1202,4 +1241,152 @@ def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float, shift: float)
     out = torch.empty((n, two_f // 2), dtype=gate_up.dtype, device=gate_up.device)
     _check(library().somi_clamped_glu(_ptr(gate_up), dtype_code(gate_up.dtype), n, two_f // 2, ctypes.c_float(limit),
                                       ctypes.c_float(alpha), ctypes.c_float(shift), _ptr(out), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ layer norm, the input convolution, normed powers
+def layernorm(h: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """(h - mean) / sqrt(var + eps) * weight + bias over float32 rows -> rows in ``out_dtype``."""
+    _need(h, "residual rows", torch.float32)
+    n, width = h.shape
+    _need(weight, "norm weight", torch.float32, (width,))
+    _need(bias, "norm bias", torch.float32, (width,))
+    out = torch.empty((n, width), dtype=out_dtype, device=h.device)
+    _check(library().somi_layernorm(_ptr(h), _ptr(weight), _ptr(bias), ctypes.c_float(eps), _ptr(out), dtype_code(out_dtype),
+                                    n, width, _stream()))
+    return out
+
+
+def layernorm_add(h: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float,
+                  copy_dtype: torch.dtype | None = None) -> torch.Tensor | None:
+    """h += layer_norm(y) * weight + bias in place on float32 rows; with ``copy_dtype`` the new rows are also returned in
+    that dtype."""
+    _need(h, "residual rows", torch.float32)
+    n, width = h.shape
+    _need(y, "rows to add", None, (n, width))
+    _need(weight, "norm weight", torch.float32, (width,))
+    _need(bias, "norm bias", torch.float32, (width,))
+    copy = torch.empty(h.shape, dtype=copy_dtype, device=h.device) if copy_dtype is not None else None
+    _check(library().somi_layernorm_add(_ptr(h), _ptr(y), dtype_code(y.dtype), _ptr(weight), _ptr(bias), ctypes.c_float(eps),
+                                        _ptr(copy), dtype_code(copy_dtype) if copy_dtype is not None else 0, n, width,
+                                        _stream()))
+    return copy
+
+
+CONV_MAX_TAPS = 9
+
+
+def input_conv(h: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, step, out_dtype: torch.dtype) -> torch.Tensor:
+    """h + conv(h) over time per channel -> [N, C] in ``out_dtype``.  h: [N, C] float32 rows of the step; taps: [C, taps]
+    float32, the last tap on the current token; state: [slots, max(taps - 1, 1), C] float32, a request's last inputs,
+    read and then advanced by the step's entries."""
+    _need(h, "residual rows", torch.float32)
+    n, channels = h.shape
+    _need(taps, "convolution taps", torch.float32)
+    if taps.dim() != 2 or taps.shape[0] != channels or not 1 <= taps.shape[1] <= CONV_MAX_TAPS:
+        raise KernelError(f"input_conv: taps {tuple(taps.shape)} != [{channels}, 1..{CONV_MAX_TAPS}]")
+    width = taps.shape[1]
+    _need(state, "convolution state", torch.float32)
+    if tuple(state.shape[1:]) != (max(width - 1, 1), channels):
+        raise KernelError(f"input_conv: state {tuple(state.shape)} != [slots, {max(width - 1, 1)}, {channels}]")
+    entries = step.state_slots.numel()
+    _need(step.token_entry, "token entries", torch.int32, (n,))
+    _need(step.entry_start, "entry offsets", torch.int32, (entries + 1,))
+    out = torch.empty((n, channels), dtype=out_dtype, device=h.device)
+    _check(library().somi_input_conv(_ptr(h), _ptr(taps), width, _ptr(state), _ptr(step.token_entry), _ptr(step.entry_start),
+                                     _ptr(step.state_slots), n, entries, channels, _ptr(out), dtype_code(out_dtype),
+                                     _stream()))
+    return out
+
+
+def poly_norm(z: torch.Tensor, coefficients: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """a N(z) + b N(z^2) + c N(z^3) + e per row with N the division by the row's root mean square; z: [N, F] float32;
+    coefficients: (a, b, c, e) float32 on the device."""
+    _need(z, "rows", torch.float32)
+    _need(coefficients, "coefficients", torch.float32, (4,))
+    out = torch.empty(z.shape, dtype=out_dtype, device=z.device)
+    _check(library().somi_poly_norm(_ptr(z), _ptr(coefficients), ctypes.c_float(eps), _ptr(out), dtype_code(out_dtype),
+                                    z.shape[0], z.shape[1], _stream()))
+    return out
+
+
+# ------------------------------------------------------------------------------------------ attention over a latent
+def head_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t, h, :] = weight[h] x[t, h, :].  x: [N, heads, K] (a view whose last dimension is contiguous); weight:
+    [heads, n_out, K]; out: [N, heads, n_out], likewise a view if given."""
+    heads, n_out, k = weight.shape
+    _need(weight, "per-head matrices", x.dtype)
+    if not x.is_cuda or x.dim() != 3 or x.shape[1] != heads or x.shape[2] != k or x.stride(2) != 1:
+        raise KernelError(f"head_linear: rows {tuple(x.shape)} do not fit matrices {tuple(weight.shape)}")
+    n = x.shape[0]
+    if out is None:
+        out = torch.empty((n, heads, n_out), dtype=x.dtype, device=x.device)
+    if out.dtype != x.dtype or tuple(out.shape) != (n, heads, n_out) or out.stride(2) != 1:
+        raise KernelError(f"head_linear: the result must be [{n}, {heads}, {n_out}] of {x.dtype}")
+    _check(library().somi_head_linear(_ptr(x), ctypes.c_int64(x.stride(0)), ctypes.c_int64(x.stride(1)), _ptr(weight),
+                                      dtype_code(x.dtype), n, heads, n_out, k, _ptr(out), ctypes.c_int64(out.stride(0)),
+                                      ctypes.c_int64(out.stride(1)), _stream()))
+    return out
+
+
+def latent_prepare(rows: torch.Tensor, q_rank: int, rank: int, rot: int, q_weight: torch.Tensor,
+                   c_weight: torch.Tensor | None, eps: float, inv_freq: torch.Tensor | None, rot_dims: int, amplitude: float,
+                   positions: torch.Tensor, slots: torch.Tensor | None, latent: torch.Tensor | None,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """From float32 rows [query latent (q_rank) | latent as projected (rank) | shared key part (rot)]: the RMS-normed
+    query latent -> [N, q_rank] in ``out_dtype``; and, with ``latent`` ([pages, page, rank + rot]), the RMS-normed
+    latent and the rotated key part into the tokens' slots."""
+    _need(rows, "projected rows", torch.float32)
+    n = rows.shape[0]
+    _need(q_weight, "query latent's norm weight", torch.float32, (q_rank,))
+    _need(positions, "positions", torch.int32, (n,))
+    if latent is not None:
+        _need(latent, "kept latents", out_dtype)
+        if latent.dim() != 3 or latent.shape[2] != rank + rot:
+            raise KernelError(f"latent_prepare: cache shape {tuple(latent.shape)} != [pages, page, {rank + rot}]")
+        _need(c_weight, "latent's norm weight", torch.float32, (rank,))
+        _need(slots, "slot mapping", torch.int32, (n,))
+        if rot_dims:
+            _need(inv_freq, "rotation frequencies", torch.float32, (rot_dims // 2,))
+    q_latent = torch.empty((n, q_rank), dtype=out_dtype, device=rows.device)
+    _check(library().somi_latent_prepare(_ptr(rows), ctypes.c_int64(rows.stride(0)), n, int(q_rank), int(rank), int(rot),
+                                         _ptr(q_weight), _ptr(c_weight), ctypes.c_float(eps), _ptr(inv_freq), int(rot_dims),
+                                         ctypes.c_float(amplitude), _ptr(positions), _ptr(slots), _ptr(q_latent),
+                                         _ptr(latent), dtype_code(out_dtype), _stream()))
+    return q_latent
+
+
+def latent_place(q: torch.Tensor, heads: int, dim: int, rot: int, rank: int, inv_freq: torch.Tensor | None, rot_dims: int,
+                 amplitude: float, positions: torch.Tensor, queries: torch.Tensor) -> None:
+    """The rotated part of every head of q ([N, heads * (dim + rot)], head by head [dim | rot]) turned by its position
+    and written to ``queries[t, h, rank:]`` ([N, heads, rank + rot])."""
+    _need(q, "projected queries", None, (queries.shape[0], heads * (dim + rot)))
+    _need(queries, "query rows", q.dtype, (q.shape[0], heads, rank + rot))
+    _need(positions, "positions", torch.int32, (q.shape[0],))
+    if rot_dims:
+        _need(inv_freq, "rotation frequencies", torch.float32, (rot_dims // 2,))
+    _check(library().somi_latent_place(_ptr(q), dtype_code(q.dtype), q.shape[0], int(heads), int(dim), int(rot), int(rank),
+                                       _ptr(inv_freq), int(rot_dims), ctypes.c_float(amplitude), _ptr(positions),
+                                       _ptr(queries), _stream()))
+
+
+def latent_attention_plain(queries: torch.Tensor, latent: torch.Tensor, block_table: torch.Tensor, token_entry: torch.Tensor,
+                           positions: torch.Tensor, rank: int, scale: float, sink: torch.Tensor) -> torch.Tensor:
+    """Causal softmax attention with a sink over kept latents: queries [N, heads, rank + rot] against the rows of
+    ``latent`` ([pages, page, rank + rot]) of each token's request up to its own position; the values are the rows' first
+    ``rank`` channels -> [N, heads, rank]."""
+    _need(queries, "query rows")
+    n, heads, width = queries.shape
+    _need(latent, "kept latents", queries.dtype)
+    if latent.dim() != 3 or latent.shape[2] != width or not 0 < rank <= width:
+        raise KernelError(f"latent_attention: cache {tuple(latent.shape)} does not fit queries of {width} (rank {rank})")
+    _need(block_table, "block table", torch.int32)
+    _need(token_entry, "token entries", torch.int32, (n,))
+    _need(positions, "positions", torch.int32, (n,))
+    _need(sink, "sinks", torch.float32, (heads,))
+    out = torch.empty((n, heads, rank), dtype=queries.dtype, device=queries.device)
+    _check(library().somi_latent_attention_plain(_ptr(queries), dtype_code(queries.dtype), _ptr(latent), _ptr(block_table),
+                                                 block_table.shape[1], _ptr(token_entry), _ptr(positions), n, heads,
+                                                 int(rank), width - int(rank), latent.shape[1], ctypes.c_float(scale),
+                                                 _ptr(sink), _ptr(out), _stream()))
     return out

@@ -4,8 +4,9 @@ from .decoder import DecoderModel
 from .loader import load_model, make_runner, make_runtime, random_model
 from .plan import LayerSpec, ModelPlan, collect_weight_specs
 from .kamedra import kamedra_plan
+from .metitar import metitar_plan
 from .qwen2 import qwen2_plan
 from .rusolorn import rusolorn_plan
 
 __all__ = ["DecoderModel", "LayerSpec", "ModelPlan", "collect_weight_specs", "load_model",
-           "kamedra_plan", "make_runner", "make_runtime", "qwen2_plan", "random_model", "rusolorn_plan"]
+           "kamedra_plan", "make_runner", "metitar_plan", "make_runtime", "qwen2_plan", "random_model", "rusolorn_plan"]

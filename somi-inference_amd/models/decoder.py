@@ -93,10 +93,7 @@ class DecoderModel:
         run whose cache it reads, or None."""
         needs: list[PagedSpec | FixedStateSpec | int | None] = []
         for run, index in enumerate(self.order):
-            if run in self.plan.cache_from:
-                needs.append(self.plan.cache_from[run])
-            else:
-                needs.append(self.layers[index].mixer.cache_spec())
+            needs.append(self.layers[index].cache_spec(self.plan.cache_from.get(run)))
         return needs
 
     # ------------------------------------------------------------------ forward

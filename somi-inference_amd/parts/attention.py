@@ -68,6 +68,8 @@ class GroupedQueryAttention(Mixer):
         self.position = build_part("position", position, prefix=self.name(self.names["position"]))
         if getattr(self.position, "pairing", "half") != "half":
             raise ValueError(f"{prefix}: this part's kernels rotate channel j with j + rotary_dim / 2 only")
+        if getattr(self.position, "amplitude", 1.0) != 1.0:
+            raise ValueError(f"{prefix}: this part's kernels take no amplitude on the rotation's cosines and sines")
 
     ROLES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj", "position": "rotary_emb",
              "q_norm": "q_norm.weight", "k_norm": "k_norm.weight"}

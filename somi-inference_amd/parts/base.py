@@ -131,12 +131,22 @@ class CompositeSpec:
     anything.  The cache manager builds each as it would for a layer of its own (paged ones join the groups of
     their window and page size, fixed state gets the request's slot) and hands them out as ``LayerCache.children``."""
 
-    parts: tuple[tuple[str, "PagedSpec | FixedStateSpec | CompositeSpec"], ...]
+    parts: tuple[tuple[str, "PagedSpec | FixedStateSpec | CompositeSpec | BorrowedCache"], ...]
 
     def __post_init__(self) -> None:
         names = [name for name, _ in self.parts]
         if not names or len(set(names)) != len(names):
             raise ValueError(f"a composite cache needs at least one part and distinct names, got {names}")
+
+
+@dataclass(frozen=True)
+class BorrowedCache:
+    """What an earlier run of a layer keeps (or, with ``path``, one named part of its composite), read and never
+    written by the run that names it.  A whole run's need may be just the earlier run's index; inside a composite a
+    part is borrowed with this, so that a layer can keep state of its own beside pages that another layer writes."""
+
+    run: int
+    path: tuple[str, ...] = ()
 
 
 def paged_specs(need) -> list[PagedSpec]:
@@ -226,6 +236,11 @@ class Norm(Part):
         ops.residual_add(h, delta)
         return self.forward(h)
 
+    def add_normed(self, h: torch.Tensor, y: torch.Tensor, copy_dtype: torch.dtype | None = None) -> torch.Tensor | None:
+        """h += norm(y) in place on the float32 residual rows, for arrangements that norm a sublayer's output instead of
+        its input; with ``copy_dtype`` the new rows are also returned in that dtype.  Norms that offer it override it."""
+        raise NotImplementedError(f"{type(self).__name__} does not norm a sublayer's output")
+
 
 class PositionEncoding(Part):
     def rotation_table(self) -> tuple[torch.Tensor, int] | None:
@@ -272,6 +287,12 @@ class Block(Part):
 
     def parts(self) -> list[Part]:
         raise NotImplementedError
+
+    def cache_spec(self, borrow_from: int | None = None):
+        """What a run of the layer keeps per request: the mixer's need, or the index of the earlier run whose cache the
+        mixer reads instead (``borrow_from``).  An arrangement that keeps something of its own beside the mixer's
+        returns a composite of both."""
+        return borrow_from if borrow_from is not None else self.mixer.cache_spec()
 
     def weight_specs(self) -> list[WeightSpec]:
         specs: list[WeightSpec] = []

@@ -57,6 +57,8 @@ class DifferentialAttention(Mixer):
         self.shares_cache = bool(shares_cache)
         self.reader_masks = tuple((int(w) if w else None, int(k)) for w, k in reader_masks)
         self.position = build_part("position", position, prefix=self.name(self.names["position"]))
+        if getattr(self.position, "amplitude", 1.0) != 1.0:
+            raise ValueError(f"{prefix}: this part's kernels take no amplitude on the rotation's cosines and sines")
         self.lam = 0.0
 
     # ------------------------------------------------------------------ weights

@@ -43,18 +43,19 @@ class TokenEmbedding(Part):
 
 
 class LMHead(Part):
-    """logits = x . W^T in float32, for the rows that were asked for only; with ``softcap`` c the logits are then
-    bounded smoothly, c * tanh(logits / c)."""
+    """logits = x . W^T in float32, for the rows that were asked for only, times ``scale`` if there is one; with
+    ``softcap`` c the logits are then bounded smoothly, c * tanh(logits / c)."""
     graph_safe = True
 
     def __init__(self, prefix: str, vocab_size: int, hidden_size: int, tied: bool = False,
-                 softcap: float | None = None, tensor: str = "weight") -> None:
+                 softcap: float | None = None, tensor: str = "weight", scale: float | None = None) -> None:
         super().__init__(prefix)
         self.vocab_size, self.hidden_size, self.tied = int(vocab_size), int(hidden_size), bool(tied)
         self.softcap = float(softcap) if softcap else None
         if self.softcap is not None and not self.softcap > 0.0:
             raise ValueError(f"{prefix}: a soft cap must be > 0, got {softcap}")
         self.tensor = str(tensor)
+        self.scale = float(scale) if scale is not None and float(scale) != 1.0 else None
         self.weight: torch.Tensor | None = None
 
     def weight_specs(self) -> list[WeightSpec]:
@@ -76,6 +77,8 @@ class LMHead(Part):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         logits = linear_kernels.linear(x, self.weight, None, torch.float32)
+        if self.scale is not None:
+            ops.scale_(logits, self.scale)
         if self.softcap is not None:
             ops.softcap_(logits, self.softcap)
         return logits

@@ -7,7 +7,7 @@ import torch
 from ..kernels import linear as linear_kernels
 from ..kernels import ops
 from ..kernels.stages import stage
-from ..weights.spec import MATRIX, WeightSpec
+from ..weights.spec import MATRIX, VECTOR, Init, WeightSpec
 from .base import FeedForward, Fetch, Runtime
 from .linear import NormedRows, Projection
 
@@ -95,3 +95,52 @@ class SwiGLU(FeedForward):
             if self.activation == "silu":
                 return self.down.deferred(ops.silu_mul(projected, block=self.INTERLEAVE))
             return self.down.deferred(ops.act_mul(projected, self.activation, block=self.INTERLEAVE))
+
+
+class PolyNormFF(FeedForward):
+    """y = down(act(up(x))) without a gate, act a polynomial of normed powers with four learned numbers (a, b, c, e):
+
+        act(z) = a N(z) + b N(z^2) + c N(z^3) + e,      N(u) = u / sqrt(mean(u^2) + eps) over a token's values,
+
+    powers taken element by element.  The up product leaves float32 sums, the three mean squares are float32, the
+    activation is rounded once to the compute dtype."""
+    graph_safe = True
+
+    ROLES = {"up": "up", "down": "down", "act": "act"}
+
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, eps: float,
+                 names: dict[str, str] | None = None, suffix: str = "weight") -> None:
+        super().__init__(prefix)
+        unknown = set(names or {}) - set(self.ROLES)
+        if unknown:
+            raise ValueError(f"{prefix}: unknown tensor roles {sorted(unknown)}; known: {sorted(self.ROLES)}")
+        self.names = {**self.ROLES, **(names or {})}
+        self.suffix = str(suffix)
+        self.hidden_size, self.intermediate_size, self.eps = int(hidden_size), int(intermediate_size), float(eps)
+
+    def _tensor(self, role: str) -> str:
+        return self.name(f"{self.names[role]}.{self.suffix}" if self.suffix else self.names[role])
+
+    def weight_specs(self) -> list[WeightSpec]:
+        h, i = self.hidden_size, self.intermediate_size
+        return [WeightSpec(self._tensor("up"), (i, h), MATRIX), WeightSpec(self._tensor("down"), (h, i), MATRIX),
+                WeightSpec(self.name(self.names["act"]), (4,), VECTOR, Init(0.3, 0.3))]
+
+    def load(self, fetch: Fetch, runtime: Runtime) -> None:
+        super().load(fetch, runtime)
+        self.up = Projection(fetch(self._tensor("up")), label="up")
+        self.down = Projection(fetch(self._tensor("down")), label="down")
+        self.coefficients = fetch(self.name(self.names["act"]))
+
+    def flops(self, tokens: int, attended: int) -> float:
+        return self.up.flops(tokens) + self.down.flops(tokens)
+
+    def forward(self, x, step=None):
+        if hasattr(x, "materialize"):
+            x = x.materialize()
+        with stage(self.up.label):
+            z = linear_kernels.linear(x, self.up.weight, None, torch.float32)
+        with stage("activation"):
+            a = ops.poly_norm(z, self.coefficients, self.eps, self.runtime.dtype)
+        with stage(self.down.label):
+            return linear_kernels.linear(a, self.down.weight, None, torch.float32)

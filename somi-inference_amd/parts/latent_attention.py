@@ -1,0 +1,148 @@
+"""Attention over a shared low-rank latent, with a sink in the softmax.
+
+Per token the layer keeps ONE vector for all heads: ``[c | r]`` with ``c = rms_norm(W_dkv h)[:rank] * w`` the latent
+and ``r`` the last ``rot`` rows of ``W_dkv h``, rotated by the token's position: a key part that all heads share.  A
+head's key is ``[U_h c | r]`` and its value ``V_h c``; queries come through a latent of their own, ``q = W_uq
+(rms_norm(W_dq h) * w_q)``, head by head ``[dim plain | rot rotated]``.  With the configuration's ``scale``,
+
+    score(i, j) = scale * (q_plain(i) . U_h c(j) + q_rot(i) . r(j)),      j <= i,
+    p(i, j)     = exp(score(i, j)) / (sum_j' exp(score(i, j')) + exp(sink_h)),
+    o_h(i)      = V_h sum_j p(i, j) c(j),
+
+then ``W_o`` on the concatenated heads.  The sink is a learned number per head that only stands in the denominator.
+Because U_h and V_h are linear, the kernels never expand keys or values: ``a_h = U_h^T q_plain`` is computed per query
+(a per-head product), the attention runs on the kept vectors themselves (one key/value head of ``rank + rot`` key
+channels whose first ``rank`` are the values), and V_h is applied to the weighted sum.  Norms, angles, scores and
+softmax are float32 in both engines.
+
+A layer that ``shares_cache`` has no W_dkv: it reads the vectors an earlier layer kept (the plan's ``cache_from``) with
+its own U, V, queries and sink.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import linear as linear_kernels
+from ..kernels import ops
+from ..kernels.stages import stage
+from ..weights.spec import MATRIX, VECTOR, Init, WeightSpec
+from .base import PAGE, Fetch, LayerCache, Mixer, PagedSpec, PageTensor, PartSpec, Runtime
+from .linear import Projection
+from .registry import build_part
+
+
+class LatentAttention(Mixer):
+    graph_safe = True
+
+    ROLES = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv",
+             "sink": "sink", "o": "o", "position": "rotary_emb"}
+
+    def __init__(self, prefix: str, hidden_size: int, num_heads: int, dim: int, rot_dim: int, value_dim: int, kv_rank: int,
+                 q_rank: int, scale: float, eps: float, position: PartSpec, shares_cache: bool = False,
+                 page_size: int | None = None, names: dict[str, str] | None = None, suffix: str = "weight") -> None:
+        """``position``: the rotation of the ``rot_dim`` channels (a rotary encoding of head size ``rot_dim``, or none).
+        ``names``: role -> the checkpoint's name under the prefix (``dq_norm``, ``dkv_norm`` and ``sink`` are whole
+        names; the matrices are followed by ``suffix`` unless it is empty)."""
+        super().__init__(prefix)
+        unknown = set(names or {}) - set(self.ROLES)
+        if unknown:
+            raise ValueError(f"{prefix}: unknown tensor roles {sorted(unknown)}; known: {sorted(self.ROLES)}")
+        self.names = {**self.ROLES, **(names or {})}
+        self.suffix = str(suffix)
+        self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
+        self.dim, self.rot_dim, self.value_dim = int(dim), int(rot_dim), int(value_dim)
+        self.kv_rank, self.q_rank = int(kv_rank), int(q_rank)
+        self.scale, self.eps = float(scale), float(eps)
+        self.shares_cache = bool(shares_cache)
+        self.page_size = int(page_size) if page_size else None
+        self.position = build_part("position", position, prefix=self.name(self.names["position"]))
+        if getattr(self.position, "pairing", "half") != "half":
+            raise ValueError(f"{prefix}: this part's kernels rotate channel j with j + rotary_dim / 2 only")
+        self.rot_dims = int(getattr(self.position, "rotary_dim", 0))
+        if self.rot_dims > self.rot_dim:
+            raise ValueError(f"{prefix}: {self.rot_dims} rotated channels do not fit a key part of {self.rot_dim}")
+
+    # ------------------------------------------------------------------ weights
+    def _matrix(self, role: str) -> str:
+        return self.name(f"{self.names[role]}.{self.suffix}" if self.suffix else self.names[role])
+
+    def weight_specs(self) -> list[WeightSpec]:
+        h, heads, rank = self.hidden_size, self.num_heads, self.kv_rank
+        specs = [
+            WeightSpec(self._matrix("dq"), (self.q_rank, h), MATRIX),
+            WeightSpec(self.name(self.names["dq_norm"]), (self.q_rank,), VECTOR, Init(1.0, 0.1)),
+            WeightSpec(self._matrix("uq"), (heads * (self.dim + self.rot_dim), self.q_rank), MATRIX),
+        ]
+        if not self.shares_cache:
+            specs += [WeightSpec(self._matrix("dkv"), (rank + self.rot_dim, h), MATRIX),
+                      WeightSpec(self.name(self.names["dkv_norm"]), (rank,), VECTOR, Init(1.0, 0.1))]
+        specs += [
+            WeightSpec(self._matrix("uk"), (heads * self.dim, rank), MATRIX),
+            WeightSpec(self._matrix("uv"), (heads * self.value_dim, rank), MATRIX),
+            WeightSpec(self.name(self.names["sink"]), (heads,), VECTOR, Init(0.0, 1.0)),
+            WeightSpec(self._matrix("o"), (h, heads * self.value_dim), MATRIX),
+        ]
+        return specs + self.position.weight_specs()
+
+    def load(self, fetch: Fetch, runtime: Runtime) -> None:
+        super().load(fetch, runtime)
+        self.position.load(fetch, runtime)
+        down = [fetch(self._matrix("dq"))] + ([] if self.shares_cache else [fetch(self._matrix("dkv"))])
+        self.down = Projection.stacked(down, label="dq/dkv")
+        self.q_norm = fetch(self.name(self.names["dq_norm"]))
+        self.c_norm = None if self.shares_cache else fetch(self.name(self.names["dkv_norm"]))
+        self.up_q = Projection(fetch(self._matrix("uq")), label="uq")
+        heads, rank = self.num_heads, self.kv_rank
+        # U_h^T per head, [heads, rank, dim]: the query's plain part goes to the latent's side
+        self.key_maps = fetch(self._matrix("uk")).view(heads, self.dim, rank).transpose(1, 2).contiguous()
+        self.value_maps = fetch(self._matrix("uv")).view(heads, self.value_dim, rank).contiguous()
+        self.sink = fetch(self.name(self.names["sink"]))
+        self.out = Projection(fetch(self._matrix("o")), label="o")
+        table = self.position.rotation_table() if self.rot_dims else None
+        self.inv_freq = table[0] if table is not None else None
+        self.amplitude = float(getattr(self.position, "amplitude", 1.0))
+
+    def flops(self, tokens: int, attended: int) -> float:
+        heads, rank = self.num_heads, self.kv_rank
+        per_head = 2.0 * tokens * heads * rank * (self.dim + self.value_dim)
+        attention = 2.0 * attended * heads * (2 * rank + self.rot_dim)
+        return self.down.flops(tokens) + self.up_q.flops(tokens) + per_head + attention + self.out.flops(tokens)
+
+    # -------------------------------------------------------------------- cache
+    def cache_spec(self) -> PagedSpec:
+        return PagedSpec((PageTensor("latent", (PAGE, self.kv_rank + self.rot_dim)),), None, self.page_size)
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, x, step, cache: LayerCache | None):
+        if cache is None or "latent" not in cache.tensors:
+            raise ValueError(f"{self.prefix}: latent attention needs a paged cache of latents")
+        if cache.writes == self.shares_cache:
+            raise ValueError(f"{self.prefix}: a layer keeps latents of its own or reads another layer's, not both")
+        if hasattr(x, "materialize"):
+            x = x.materialize()
+        view = step.paged[cache.group]
+        latent = cache.tensors["latent"]
+        heads, rank, rot, dtype = self.num_heads, self.kv_rank, self.rot_dim, self.runtime.dtype
+        n = x.shape[0]
+        with stage(self.down.label):
+            rows = linear_kernels.linear(x, self.down.weight, None, torch.float32)
+        with stage("latent norms, rotation, cache write"):
+            q_latent = ops.latent_prepare(rows, self.q_rank, rank, rot, self.q_norm, self.c_norm, self.eps, self.inv_freq,
+                                          self.rot_dims, self.amplitude, step.positions,
+                                          None if self.shares_cache else view.slot_mapping,
+                                          None if self.shares_cache else latent, dtype)
+        q = self.up_q(q_latent)
+        with stage("queries to the latent's side"):
+            queries = torch.empty((n, heads, rank + rot), dtype=dtype, device=q.device)
+            ops.head_linear(q.view(n, heads, self.dim + rot)[:, :, :self.dim], self.key_maps, out=queries[:, :, :rank])
+            if rot:
+                ops.latent_place(q, heads, self.dim, rot, rank, self.inv_freq, self.rot_dims, self.amplitude,
+                                 step.positions, queries)
+        with stage("attention"):
+            mixed = ops.latent_attention_plain(queries, latent, view.block_table, step.token_entry, step.positions,
+                                               rank, self.scale, self.sink)
+        with stage("values from the latent"):
+            values = ops.head_linear(mixed, self.value_maps).view(n, heads * self.value_dim)
+        with stage(self.out.label):
+            return linear_kernels.linear(values, self.out.weight, None, torch.float32)

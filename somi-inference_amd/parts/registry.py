@@ -11,7 +11,7 @@ from typing import Any
 
 from .base import PartSpec
 
-CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head", "token_input")
+CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head", "token_input", "input_conv")
 _PARTS: dict[str, dict[str, type]] = {c: {} for c in CATEGORIES}
 
 
