@@ -114,6 +114,12 @@ class LatentAttention(Mixer):
         return PagedSpec((PageTensor("latent", (PAGE, self.kv_rank + self.rot_dim)),), None, self.page_size)
 
     # ------------------------------------------------------------------ forward
+    def attend(self, queries: torch.Tensor, latent: torch.Tensor, step, view) -> torch.Tensor:
+        """The weighted sums of the kept latents for ``queries`` [N, heads, rank + rot] (the plain part already on the
+        latent's side) -> [N, heads, rank]."""
+        return ops.latent_attention_plain(queries, latent, view.block_table, step.token_entry, step.positions,
+                                          self.kv_rank, self.scale, self.sink)
+
     def forward(self, x, step, cache: LayerCache | None):
         if cache is None or "latent" not in cache.tensors:
             raise ValueError(f"{self.prefix}: latent attention needs a paged cache of latents")
@@ -140,8 +146,7 @@ class LatentAttention(Mixer):
                 ops.latent_place(q, heads, self.dim, rot, rank, self.inv_freq, self.rot_dims, self.amplitude,
                                  step.positions, queries)
         with stage("attention"):
-            mixed = ops.latent_attention_plain(queries, latent, view.block_table, step.token_entry, step.positions,
-                                               rank, self.scale, self.sink)
+            mixed = self.attend(queries, latent, step, view)
         with stage("values from the latent"):
             values = ops.head_linear(mixed, self.value_maps).view(n, heads * self.value_dim)
         with stage(self.out.label):

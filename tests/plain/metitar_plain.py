@@ -157,9 +157,12 @@ def routing(h: torch.Tensor, weights: dict, prefix: str, mlp: dict) -> tuple[tor
     return order[:, :top], ranked[:, :top], margin
 
 
-def routed_experts(h: torch.Tensor, weights: dict, prefix: str, mlp: dict) -> torch.Tensor:
-    """sum over the chosen experts of expert(w h): the weight multiplies the expert's input; plus the shared expert."""
-    chosen, weight, _ = routing(h, weights, prefix, mlp)
+def routed_experts(h: torch.Tensor, weights: dict, prefix: str, mlp: dict, margins: list | None = None) -> torch.Tensor:
+    """sum over the chosen experts of expert(w h): the weight multiplies the expert's input; plus the shared expert.
+    ``margins`` collects, per layer, how far each token's choice is from a tie."""
+    chosen, weight, margin = routing(h, weights, prefix, mlp)
+    if margins is not None:
+        margins.append(margin)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, w in zip(chosen[t].tolist(), weight[t]):
@@ -177,7 +180,7 @@ def token_input(x: torch.Tensor, tokens: torch.Tensor, weights: dict, index: int
 
 
 # ------------------------------------------------------------------------------------- the model
-def forward(tokens, weights: dict, config: dict, want_layers: bool = False):
+def forward(tokens, weights: dict, config: dict, want_layers: bool = False, margins: list | None = None):
     """Logits [T, vocab] of one whole sequence; with ``want_layers`` also the residual stream after every layer."""
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     eps = config["norm"]["eps"]
@@ -205,7 +208,7 @@ def forward(tokens, weights: dict, config: dict, want_layers: bool = False):
             if mlp["kind"] == "dense":
                 y = poly_norm_ff(x, weights, p + ".mlp", eps)
             else:
-                y = routed_experts(x, weights, p + ".mlp", mlp)
+                y = routed_experts(x, weights, p + ".mlp", mlp, margins)
             x = x + layer_norm(y, weights, p + ".norm2", eps)
         if side:
             x = x + token_input(x, tokens, weights, index, side["dim"], eps)
