@@ -121,6 +121,57 @@ def rusolorn_closest_config_dict(sizes: str) -> dict:
             "layers": [recurrent, attention] * (RUSOLORN_LAYERS // 2)}
 
 
+# layer sizes of Metitar models that resemble real ones: (width, attention heads, unrotated and rotated query/key
+# channels a head, value size, latent size, query latent size, recurrent heads, their key size, their value size, taps,
+# experts, experts a token, an expert's size, the shared expert's size, the dense feed-forward's size, columns of the
+# token input, vocabulary).  Six layers: attention over the latent with a dense feed-forward, two recurrent layers with
+# experts and a dense feed-forward, attention with experts, a recurrent layer with experts, attention that reads the
+# fourth layer's latent with a dense feed-forward.
+METITAR_SIZES = {
+    "1b": (2048, 16, 128, 64, 128, 512, 768, 16, 128, 128, 4, 32, 4, 512, 1024, 4096, 128, 32000),
+    "7b": (4096, 32, 128, 64, 128, 512, 1536, 32, 128, 128, 4, 64, 6, 1024, 2048, 8192, 256, 32000),
+}
+METITAR_LAYERS = 6
+
+
+def metitar_config_dict(sizes: str) -> dict:
+    (width, heads, dim, rot, vdim, rank, q_rank, r_heads, r_dim, r_vdim, taps, experts, top, ff, shared, dense_ff, side,
+     vocab) = METITAR_SIZES[sizes]
+    dense = {"kind": "dense", "ff": dense_ff}
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": ff}, "shared": {"ff": shared}}
+
+    def attention(mlp, kv_from=None):
+        mixer = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "kv_rank": rank, "q_rank": q_rank,
+                 "scale": (dim + rot) ** -0.5,
+                 "rot": {"base": 10000.0, "dims": rot, "scaling": {"factor": 40.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+        if kv_from is not None:
+            mixer["kv_from"] = kv_from
+        return {"type": "latent_attention", "mixer": mixer, "mlp": mlp}
+
+    def recurrent(mlp):
+        return {"type": "hgrn2", "mixer": {"heads": r_heads, "dim": r_dim, "vdim": r_vdim}, "mlp": mlp}
+    return {"architecture": "Metitar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+            "logit_scale": 1.0, "canon": {"taps": taps}, "token_side": {"dim": side},
+            "layers": [attention(dense), recurrent(moe), recurrent(dense), attention(moe), recurrent(moe), attention(dense, 3)]}
+
+
+def metitar_closest_config_dict(sizes: str) -> dict:
+    """The closest model the engine had before: a Rusolorn model of the same width, attention heads and head size (a
+    window longer than any context here, so its attention is causal over everything as well), recurrent heads and state
+    size, experts, shared expert, token input and layers.  Each of its layers runs attention AND a recurrence and has
+    experts; a Metitar layer has one mixer and experts in half of its layers."""
+    (width, heads, dim, rot, vdim, rank, q_rank, r_heads, r_dim, r_vdim, taps, experts, top, ff, shared, dense_ff, side,
+     vocab) = METITAR_SIZES[sizes]
+    layer = {"type": "parallel",
+             "mixer": {"left": {"heads": heads, "kv_heads": heads // 4, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                "mask": {"size": 1 << 20}},
+                       "right": {"heads": r_heads, "kv_heads": r_heads // 2, "dim": r_dim, "vdim": r_vdim, "conv": taps}},
+             "mlp": {"kind": "moe", "router": {"experts": experts, "top": top, "groups": {"count": 1, "keep": 1}},
+                     "expert": {"ff": ff, "limit": 7.0}, "shared": {"ff": shared, "limit": 7.0}}}
+    return {"architecture": "Rusolorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
+            "residual_mult": 0.5, "token_side": {"dim": side}, "layers": [layer] * METITAR_LAYERS}
+
+
 # keys of a config.json that name sizes, in the order they are reported under "config" (flat, at most 20 keys)
 SIZE_KEYS = ("hidden_size", "intermediate_size", "num_attention_heads", "num_key_value_heads", "head_dim",
              "vocab_size", "tie_word_embeddings")
@@ -161,6 +212,10 @@ def parse_args() -> argparse.Namespace:
                    help="instead of the default workload: prefill and decode of a Rusolorn model (windowed attention "
                         "beside a gated delta rule, routed experts) at these layer sizes, beside the Kamedra model of "
                         "equal width, heads, active feed-forward size and layers, each with its stage times")
+    p.add_argument("--metitar", default=None, choices=sorted(METITAR_SIZES), metavar="SIZES",
+                   help="instead of the default workload: prefill and decode of a Metitar model (attention over a shared "
+                        "latent, the HGRN2 recurrence, dense and routed feed-forwards) at these layer sizes, beside the "
+                        "Rusolorn model of equal width, heads, experts and layers, each with its stage times")
     p.add_argument("--serving", type=int, default=0, metavar="REQUESTS",
                    help="also run this many requests (prompts of 128 to 2,048 tokens, 256 new tokens each) through "
                         "the scheduler with portions of 512, and report it under 'serving'")
@@ -657,6 +712,76 @@ def run_rusolorn(args) -> dict:
     return out
 
 
+def run_metitar(args) -> dict:
+    """Prefill and decode of a Metitar model beside the closest Rusolorn model, with the stage times of both and what
+    the attention, recurrence and feed-forward stages reach of the machine."""
+    (width, heads, dim, rot, vdim, rank, q_rank, r_heads, r_dim, r_vdim, taps, experts, top, ff, shared, dense_ff, side,
+     vocab) = METITAR_SIZES[args.metitar]
+    batches, context, tokens = (8, 64), args.context, args.prefill_tokens
+    out: dict = {}
+    for label, config_dict in (("metitar", metitar_config_dict(args.metitar)),
+                               ("closest", metitar_closest_config_dict(args.metitar))):
+        bench = Workbench(config_dict, dtype=args.dtype, seed=args.seed, block_size=args.block_size,
+                          pool_tokens=Workbench.pool_tokens(batches, context, tokens), max_requests=max(batches))
+        block: dict = {"prefill": {str(n): bench.prefill_run(n) for n in sorted({512, tokens})}}
+        for batch in batches:
+            run = bench.decode_run(batch, max(POINT_MIN_STEPS, args.steps // 2), max(2, args.warmup // 2), context)
+            block[f"decode_b{batch}"] = {"tok_s": round(run["tok_s"], 1), "ms": round(run["ms"], 4),
+                                        "mean_ctx": round(run["mean_ctx"], 1)}
+        block["stages"] = bench.stage_run(tokens, batches[0], context)
+        print_stage_tables(block["stages"])
+        out[label] = block
+        bench.close()
+    bf16_peak = PEAK_FLOPS["bfloat16"]
+    pairs = tokens * (tokens + 1) // 2
+
+    def stage_ms(block, run, *names):
+        return sum(block["stages"][run].get(name, {}).get("ms", 0.0) for name in names)
+
+    def rate(flops, ms):
+        return {"ms": round(ms, 4), "tflops": round(flops / 1e9 / max(ms, 1e-9), 2),
+                "frac_of_peak": round(flops / 1e3 / max(ms, 1e-9) / bf16_peak * 1e6, 5)}
+    run, layers = f"prefill_{tokens}", METITAR_LAYERS
+    attention_layers, recurrent_layers, expert_layers, dense_layers = 3, 3, 3, 3
+    out["prefill_kernels"] = {
+        "tokens": tokens,
+        # scores over the latent and the shared key part, weights times the latent, over the visible pairs
+        "metitar_attention": rate(attention_layers * 2.0 * heads * (2 * rank + rot) * pairs, stage_ms(out["metitar"], run, "attention")),
+        "closest_attention": rate(layers * 4.0 * heads * dim * pairs, stage_ms(out["closest"], run, "attention")),
+        # the per-head maps on either side of the attention (no like kernel in the closest model)
+        "metitar_head_maps": rate(attention_layers * 2.0 * tokens * heads * rank * (dim + vdim),
+                                  stage_ms(out["metitar"], run, "queries to the latent's side", "values from the latent")),
+        # per token and head: two passes over the state here (update, product), three in the closest model
+        "metitar_recurrence": rate(recurrent_layers * 4.0 * r_heads * r_dim * r_vdim * tokens, stage_ms(out["metitar"], run, "recurrence")),
+        "closest_recurrence": rate(layers * 6.0 * r_heads * r_dim * r_vdim * tokens, stage_ms(out["closest"], run, "recurrence")),
+        "metitar_experts": rate(expert_layers * 6.0 * tokens * top * ff * width,
+                                stage_ms(out["metitar"], run, "experts gate_up", "experts down")),
+        "closest_experts": rate(layers * 6.0 * tokens * top * ff * width,
+                                stage_ms(out["closest"], run, "experts gate_up", "experts down")),
+        "metitar_dense": rate(dense_layers * 4.0 * tokens * dense_ff * width, stage_ms(out["metitar"], run, "up", "down")),
+        "metitar_router": {"ms": round(stage_ms(out["metitar"], run, "router"), 4)},
+        "closest_router": {"ms": round(stage_ms(out["closest"], run, "router"), 4)},
+    }
+    run = f"decode_b{batches[0]}_eager"
+
+    def stream(bytes_, ms):
+        return {"ms": round(ms, 4), "gbs": round(bytes_ / 1e6 / max(ms, 1e-9), 1)}
+    used = min(experts, batches[0] * top)          # experts a step touches at most
+    out["decode_kernels"] = {
+        "batch": batches[0], "context": context,
+        # one kept vector a token for all heads, against keys and values for every key/value head
+        "metitar_attention": stream(attention_layers * batches[0] * context * (rank + rot) * 2.0, stage_ms(out["metitar"], run, "attention")),
+        "closest_attention": stream(layers * batches[0] * context * (heads // 4) * 2 * dim * 2.0, stage_ms(out["closest"], run, "attention")),
+        "metitar_recurrence": stream(recurrent_layers * batches[0] * r_heads * r_dim * r_vdim * 4.0 * 2, stage_ms(out["metitar"], run, "recurrence")),
+        "closest_recurrence": stream(layers * batches[0] * r_heads * r_dim * r_vdim * 4.0 * 2, stage_ms(out["closest"], run, "recurrence")),
+        "metitar_experts": stream(expert_layers * used * 3.0 * ff * width * 2.0,
+                                  stage_ms(out["metitar"], run, "experts gate_up", "experts down")),
+        "closest_experts": stream(layers * used * 3.0 * ff * width * 2.0,
+                                  stage_ms(out["closest"], run, "experts gate_up", "experts down")),
+    }
+    return out
+
+
 def main() -> int:
     args = parse_args()
     world = int(os.environ.get("WORLD_SIZE", "1"))
@@ -671,6 +796,16 @@ def main() -> int:
                 "data": "synthetic: seeded random weights, seeded uniform token ids", "sizes": args.kamedra}
         line.update(run_kamedra(args))
         line["value"] = line["kamedra"][f"decode_b8"]["tok_s"]
+        line["seconds_total"] = round(time.perf_counter() - started, 1)
+        print(json.dumps(line))
+        return 0
+
+    if args.metitar:
+        line = {"metric": f"Metitar at {args.metitar} layer sizes beside the closest Rusolorn model: prefill and decode",
+                "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                "data": "synthetic: seeded random weights, seeded uniform token ids", "sizes": args.metitar}
+        line.update(run_metitar(args))
+        line["value"] = line["metitar"]["decode_b8"]["tok_s"]
         line["seconds_total"] = round(time.perf_counter() - started, 1)
         print(json.dumps(line))
         return 0

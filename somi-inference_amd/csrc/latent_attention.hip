@@ -11,7 +11,7 @@
 // and no value; it is not scaled.  Causal: position i sees every j <= i of its request.
 //
 //   prepare   RMS norm of the query latent (rows out in the compute dtype), RMS norm of c and rotation of r into the
-//             request's pages
+//             request's pages (and c once more, transposed inside its page, where the matrix-core kernel wants it)
 //   place     a head's rotated query part goes behind its a_h in the query rows that the attention reads
 //   plain     one workgroup per (token, head), float32 online softmax over 128-key tiles aligned to absolute
 //             positions, which starts from the sink (running maximum = sink, running sum = 1, output 0)
@@ -26,7 +26,7 @@ latent_prepare_kernel(const float* __restrict__ rows, int64_t row_stride, int q_
                       const float* __restrict__ q_weight, const float* __restrict__ c_weight, float eps,
                       const float* __restrict__ inv_freq, int rot_dims, float amplitude,
                       const int* __restrict__ positions, const int* __restrict__ slots, T* __restrict__ q_latent,
-                      T* __restrict__ latent) {
+                      T* __restrict__ latent, T* __restrict__ latent_t, int page_size) {
     __shared__ float red[16];
     const int64_t t = blockIdx.x;
     const float* row = rows + t * row_stride;
@@ -44,7 +44,13 @@ latent_prepare_kernel(const float* __restrict__ rows, int64_t row_stride, int q_
     ss = block_sum<256>(ss, red);
     const float inv_c = 1.0f / sqrtf(ss / (float)rank + eps);
     T* kept = latent + (int64_t)slot * (rank + rot);
-    for (int i = threadIdx.x; i < rank; i += 256) kept[i] = from_float<T>(kv[i] * inv_c * c_weight[i]);
+    // the same latent once more, transposed inside its page ([pages, rank, page]), for kernels that read it by channel
+    T* kept_t = latent_t != nullptr ? latent_t + (int64_t)(slot / page_size) * rank * page_size + slot % page_size : nullptr;
+    for (int i = threadIdx.x; i < rank; i += 256) {
+        const T v = from_float<T>(kv[i] * inv_c * c_weight[i]);
+        kept[i] = v;
+        if (kept_t != nullptr) kept_t[(int64_t)i * page_size] = v;
+    }
     const float p = (float)positions[t];
     const int half = rot_dims / 2;
     for (int i = threadIdx.x; i < rot; i += 256) {
@@ -63,19 +69,21 @@ latent_prepare_kernel(const float* __restrict__ rows, int64_t row_stride, int q_
 extern "C" int somi_latent_prepare(const float* rows, int64_t row_stride, int n_tokens, int q_rank, int rank, int rot,
                                    const float* q_weight, const float* c_weight, float eps, const float* inv_freq,
                                    int rot_dims, float amplitude, const int* positions, const int* slots,
-                                   void* q_latent, void* latent, int dtype, hipStream_t stream) {
+                                   void* q_latent, void* latent, void* latent_t, int page_size, int dtype,
+                                   hipStream_t stream) {
     SOMI_REQUIRE(n_tokens >= 0 && q_rank > 0 && rank > 0 && rot >= 0, "latent_prepare: bad sizes");
     SOMI_REQUIRE(rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0, "latent_prepare: %d rotated channels of %d", rot_dims, rot);
     SOMI_REQUIRE(row_stride >= q_rank + (latent ? rank + rot : 0), "latent_prepare: rows too narrow");
+    SOMI_REQUIRE(latent_t == nullptr || (latent != nullptr && page_size > 0), "latent_prepare: transposed pages need the pages and their size");
     if (n_tokens == 0) return 0;
     if (dtype == SOMI_F32)
         hipLaunchKernelGGL(latent_prepare_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, rows, row_stride, q_rank,
                            rank, rot, q_weight, c_weight, eps, inv_freq, rot_dims, amplitude, positions, slots,
-                           (float*)q_latent, (float*)latent);
+                           (float*)q_latent, (float*)latent, (float*)latent_t, page_size);
     else if (dtype == SOMI_BF16)
         hipLaunchKernelGGL(latent_prepare_kernel<bf16>, dim3(n_tokens), dim3(256), 0, stream, rows, row_stride, q_rank,
                            rank, rot, q_weight, c_weight, eps, inv_freq, rot_dims, amplitude, positions, slots,
-                           (bf16*)q_latent, (bf16*)latent);
+                           (bf16*)q_latent, (bf16*)latent, (bf16*)latent_t, page_size);
     else
         return somi_fail("latent_prepare: unknown dtype %d", dtype);
     SOMI_LAUNCH_CHECK("latent_prepare");

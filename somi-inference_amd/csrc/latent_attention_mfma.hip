@@ -1,0 +1,234 @@
+// Attention over kept latents on the matrix cores (bfloat16).
+//
+// Every past token keeps one row [c (rank) | r (rot)] for all heads, and the same c once more transposed inside its
+// page ([pages, rank, page]: consecutive positions of one channel are adjacent, the operand layout of the
+// weights-times-values product).  A workgroup serves ONE token and up to 16 of its heads (its query slots), which all
+// see the same keys, over one part of the token's keys (a key split); its four wavefronts walk 64-key tiles:
+//
+//   scores   wavefront w owns keys 16 w .. 16 w + 15 of the tile: S^T = K Q^T by `16x16x32` products over the rank + rot
+//            channels, K fragments straight from the rows (16 bytes a lane), the slots' Q fragments held in registers
+//            for the whole walk; a lane then holds 4 keys of one slot
+//   softmax  float32, online: the running maximum of a slot starts at the head's sink and its running sum at 1 (the
+//            sink's own term, in the first key split only), the tile's maximum is exchanged through LDS
+//   values   the weights go to LDS as two bfloat16 halves (p = hi + lo, so no weight is rounded to eight bits) and
+//            come back as B operands; wavefront w owns the channel tiles w, w + 4, ... of the output, O^T = C^T P^T with
+//            the C^T fragments straight from the transposed pages
+//
+// A token's key splits leave (maximum, sum, unnormed output) in a workspace and a second kernel joins them.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 lam_bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 lam_bf16x4;
+typedef __attribute__((ext_vector_type(4))) float lam_f32x4;
+
+#define LAM_KEYS 64
+
+template <int STEPS, int CT>
+__global__ void __launch_bounds__(256)
+latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __restrict__ latent,
+                             const bf16* __restrict__ latent_t, const int* __restrict__ block_table, int max_blocks,
+                             const int* __restrict__ token_entry, const int* __restrict__ positions, int n_tokens,
+                             int heads, int rank, int D, int page_size, float scale, const float* __restrict__ sink,
+                             int splits, bf16* __restrict__ out, float* __restrict__ part) {
+    __shared__ float wmax[4][16];
+    __shared__ float wsum[4][16];
+    __shared__ __attribute__((aligned(16))) bf16 p_hi[16][LAM_KEYS + 8];
+    __shared__ __attribute__((aligned(16))) bf16 p_lo[16][LAM_KEYS + 8];
+    const int t = n_tokens - 1 - (int)blockIdx.x;               // the longest walks first
+    const int hg = blockIdx.y, split = blockIdx.z;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int col = lane & 15, quad = lane >> 4;
+    const int head = hg * 16 + col;
+    const bool live = head < heads;
+    const int p = positions[t];
+    const int* table = block_table + (int64_t)token_entry[t] * max_blocks;
+    const int steps = (D + 31) >> 5, tiles_c = rank >> 4;
+    // this split's keys: whole 64-key tiles of the token's p + 1 keys
+    const int tiles_all = (p + LAM_KEYS) / LAM_KEYS;
+    const int per = (tiles_all + splits - 1) / splits;
+    const int k_begin = split * per * LAM_KEYS;
+    const int k_end = min(p + 1, (split + 1) * per * LAM_KEYS);
+
+    lam_bf16x8 qf[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+        const int ch = s * 32 + quad * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) qf[s][i] = (__bf16)0.f;
+        if (s < steps && live && ch < D)
+            qf[s] = *reinterpret_cast<const lam_bf16x8*>(queries + ((int64_t)t * heads + head) * D + ch);
+    }
+    lam_f32x4 acc[CT];
+#pragma unroll
+    for (int j = 0; j < CT; ++j) acc[j] = lam_f32x4{0.f, 0.f, 0.f, 0.f};
+    float m = split == 0 ? (live ? sink[head] : 0.f) : -INFINITY;
+    float lsum = (split == 0 && w == 0 && quad == 0) ? 1.f : 0.f;
+
+    for (int kb = k_begin; kb < k_end; kb += LAM_KEYS) {
+        // ---- scores of this wavefront's 16 keys
+        const int key_row = min(kb + 16 * w + col, p);
+        const bf16* krow = latent + ((int64_t)table[key_row / page_size] * page_size + key_row % page_size) * D;
+        lam_bf16x8 kf[STEPS];
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            const int ch = s * 32 + quad * 8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) kf[s][i] = (__bf16)0.f;
+            if (s < steps && ch < D) kf[s] = *reinterpret_cast<const lam_bf16x8*>(krow + ch);
+        }
+        lam_f32x4 sc = lam_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s)
+            if (s < steps) sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[s], qf[s], sc, 0, 0, 0);
+        // ---- the transposed latents of the channel tiles this wavefront owns, asked for before the softmax
+        lam_bf16x8 vf[CT][2];
+#pragma unroll
+        for (int j = 0; j < CT; ++j) {
+            const int ct = w + 4 * j;
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) vf[j][half][i] = (__bf16)0.f;
+                if (ct < tiles_c) {
+                    const int key8 = min(kb + half * 32 + quad * 8, p & ~7);
+                    const bf16* vrow = latent_t + (((int64_t)table[key8 / page_size] * rank + ct * 16 + col) * page_size
+                                                   + key8 % page_size);
+                    vf[j][half] = *reinterpret_cast<const lam_bf16x8*>(vrow);
+                }
+            }
+        }
+        // ---- softmax over the tile, float32
+        float s4[4], mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int key = kb + 16 * w + quad * 4 + i;
+            s4[i] = key < k_end ? sc[i] * scale : -INFINITY;
+            mx = fmaxf(mx, s4[i]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        if (quad == 0) wmax[w][col] = mx;
+        __syncthreads();
+        const float m_new = fmaxf(fmaxf(m, fmaxf(wmax[0][col], wmax[1][col])), fmaxf(wmax[2][col], wmax[3][col]));
+        const float corr = __expf(m - m_new);
+        m = m_new;
+        float psum = 0.f;
+        lam_bf16x4 hi, lo;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float pv = __expf(s4[i] - m_new);              // exp(-inf) = 0 for keys that are not seen
+            psum += pv;
+            hi[i] = (__bf16)pv;
+            lo[i] = (__bf16)(pv - (float)hi[i]);
+        }
+        lsum = lsum * corr + psum;
+        *reinterpret_cast<lam_bf16x4*>(&p_hi[col][16 * w + quad * 4]) = hi;
+        *reinterpret_cast<lam_bf16x4*>(&p_lo[col][16 * w + quad * 4]) = lo;
+#pragma unroll
+        for (int j = 0; j < CT; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[j][i] *= corr;
+        __syncthreads();
+        // ---- weights times latents
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const lam_bf16x8 ph = *reinterpret_cast<const lam_bf16x8*>(&p_hi[col][half * 32 + quad * 8]);
+            const lam_bf16x8 pl = *reinterpret_cast<const lam_bf16x8*>(&p_lo[col][half * 32 + quad * 8]);
+#pragma unroll
+            for (int j = 0; j < CT; ++j)
+                if (w + 4 * j < tiles_c) {
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j][half], ph, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j][half], pl, acc[j], 0, 0, 0);
+                }
+        }
+    }
+    // ---- the slots' sums: the lane groups of a wavefront, then the wavefronts
+    lsum += __shfl_xor(lsum, 16, 64);
+    lsum += __shfl_xor(lsum, 32, 64);
+    __syncthreads();
+    if (quad == 0) wsum[w][col] = lsum;
+    __syncthreads();
+    const float l = (wsum[0][col] + wsum[1][col]) + (wsum[2][col] + wsum[3][col]);
+    if (!live) return;
+    if (splits == 1) {
+        const float inv = 1.0f / l;
+#pragma unroll
+        for (int j = 0; j < CT; ++j) {
+            const int ct = w + 4 * j;
+            if (ct >= tiles_c) continue;
+            lam_bf16x4 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[i] = (__bf16)(acc[j][i] * inv);
+            *reinterpret_cast<lam_bf16x4*>(out + ((int64_t)t * heads + head) * rank + ct * 16 + quad * 4) = o;
+        }
+        return;
+    }
+    float* mine = part + (((int64_t)t * heads + head) * splits + split) * (rank + 2);
+#pragma unroll
+    for (int j = 0; j < CT; ++j) {
+        const int ct = w + 4 * j;
+        if (ct >= tiles_c) continue;
+        *reinterpret_cast<lam_f32x4*>(mine + ct * 16 + quad * 4) = acc[j];
+    }
+    if (w == 0 && quad == 0) {
+        mine[rank] = m;
+        mine[rank + 1] = l;
+    }
+}
+
+// out[t, h, :] = sum_s exp(m_s - M) O_s / sum_s exp(m_s - M) l_s over a token's key splits (a split without keys has
+// m = -inf and weighs nothing).  One workgroup per (token, head).
+__global__ void __launch_bounds__(128)
+latent_attention_join_kernel(const float* __restrict__ part, int splits, int rank, bf16* __restrict__ out) {
+    const int64_t slot = blockIdx.x;
+    const float* mine = part + slot * splits * (rank + 2);
+    float top = -INFINITY;
+    for (int s = 0; s < splits; ++s) top = fmaxf(top, mine[s * (rank + 2) + rank]);
+    float total = 0.f;
+    for (int s = 0; s < splits; ++s) total += __expf(mine[s * (rank + 2) + rank] - top) * mine[s * (rank + 2) + rank + 1];
+    const float inv = 1.0f / total;
+    for (int c = threadIdx.x; c < rank; c += 128) {
+        float sum = 0.f;
+        for (int s = 0; s < splits; ++s) sum += __expf(mine[s * (rank + 2) + rank] - top) * mine[s * (rank + 2) + c];
+        out[slot * rank + c] = (bf16)(sum * inv);
+    }
+}
+
+extern "C" int somi_latent_attention_mfma_supported(int rank, int rot, int page_size) {
+    const int D = rank + rot;
+    return rank > 0 && rank % 16 == 0 && D % 16 == 0 && D <= 576 && rank <= 512 && page_size % 8 == 0;
+}
+
+// queries: [n_tokens, heads, rank + rot] bfloat16; latent: [pages, page, rank + rot]; latent_t: [pages, rank, page];
+// block_table: [entries, max_blocks]; sink: [heads] float32; out: [n_tokens, heads, rank] bfloat16; part: a workspace of
+// n_tokens * heads * splits * (rank + 2) floats where splits > 1.
+extern "C" int somi_latent_attention_mfma(const void* queries, const void* latent, const void* latent_t,
+                                          const int* block_table, int max_blocks, const int* token_entry,
+                                          const int* positions, int n_tokens, int heads, int rank, int rot, int page_size,
+                                          float scale, const float* sink, int splits, void* out, float* part,
+                                          hipStream_t stream) {
+    SOMI_REQUIRE(n_tokens >= 0 && heads > 0 && max_blocks > 0 && splits >= 1, "latent_attention_mfma: bad sizes");
+    SOMI_REQUIRE(somi_latent_attention_mfma_supported(rank, rot, page_size),
+                 "latent_attention_mfma: a latent of %d + %d in pages of %d is not what the kernel is built for", rank, rot,
+                 page_size);
+    SOMI_REQUIRE(splits == 1 || part != nullptr, "latent_attention_mfma: key splits need a workspace");
+    SOMI_REQUIRE(ceil_div(heads, 16) <= 65535 && splits <= 65535, "latent_attention_mfma: too many heads or splits");
+    if (n_tokens == 0) return 0;
+    const int D = rank + rot;
+    const dim3 grid(n_tokens, ceil_div(heads, 16), splits);
+#define LAM_LAUNCH(STEPS, CT)                                                                                          \
+    hipLaunchKernelGGL((latent_attention_mfma_kernel<STEPS, CT>), grid, dim3(256), 0, stream, (const bf16*)queries,     \
+                       (const bf16*)latent, (const bf16*)latent_t, block_table, max_blocks, token_entry, positions,    \
+                       n_tokens, heads, rank, D, page_size, scale, sink, splits, (bf16*)out, part)
+    if (D <= 128 && rank <= 128) LAM_LAUNCH(4, 2);
+    else if (D <= 256 && rank <= 256) LAM_LAUNCH(8, 4);
+    else LAM_LAUNCH(18, 8);
+#undef LAM_LAUNCH
+    SOMI_LAUNCH_CHECK("latent_attention_mfma");
+    if (splits > 1) {
+        hipLaunchKernelGGL(latent_attention_join_kernel, dim3((unsigned)((int64_t)n_tokens * heads)), dim3(128), 0, stream,
+                           part, splits, rank, (bf16*)out);
+        SOMI_LAUNCH_CHECK("latent_attention_join");
+    }
+    return 0;
+}

@@ -1332,10 +1332,11 @@ def head_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None 
 def latent_prepare(rows: torch.Tensor, q_rank: int, rank: int, rot: int, q_weight: torch.Tensor,
                    c_weight: torch.Tensor | None, eps: float, inv_freq: torch.Tensor | None, rot_dims: int, amplitude: float,
                    positions: torch.Tensor, slots: torch.Tensor | None, latent: torch.Tensor | None,
-                   out_dtype: torch.dtype) -> torch.Tensor:
+                   out_dtype: torch.dtype, latent_t: torch.Tensor | None = None) -> torch.Tensor:
     """From float32 rows [query latent (q_rank) | latent as projected (rank) | shared key part (rot)]: the RMS-normed
     query latent -> [N, q_rank] in ``out_dtype``; and, with ``latent`` ([pages, page, rank + rot]), the RMS-normed
-    latent and the rotated key part into the tokens' slots."""
+    latent and the rotated key part into the tokens' slots (``latent_t`` [pages, rank, page]: the latent once more,
+    transposed inside its page)."""
     _need(rows, "projected rows", torch.float32)
     n = rows.shape[0]
     _need(q_weight, "query latent's norm weight", torch.float32, (q_rank,))
@@ -1348,11 +1349,16 @@ def latent_prepare(rows: torch.Tensor, q_rank: int, rank: int, rot: int, q_weigh
         _need(slots, "slot mapping", torch.int32, (n,))
         if rot_dims:
             _need(inv_freq, "rotation frequencies", torch.float32, (rot_dims // 2,))
+        if latent_t is not None:
+            _need(latent_t, "transposed latents", out_dtype, (latent.shape[0], rank, latent.shape[1]))
+    elif latent_t is not None:
+        raise KernelError("latent_prepare: transposed pages without the pages")
     q_latent = torch.empty((n, q_rank), dtype=out_dtype, device=rows.device)
     _check(library().somi_latent_prepare(_ptr(rows), ctypes.c_int64(rows.stride(0)), n, int(q_rank), int(rank), int(rot),
                                          _ptr(q_weight), _ptr(c_weight), ctypes.c_float(eps), _ptr(inv_freq), int(rot_dims),
                                          ctypes.c_float(amplitude), _ptr(positions), _ptr(slots), _ptr(q_latent),
-                                         _ptr(latent), dtype_code(out_dtype), _stream()))
+                                         _ptr(latent), _ptr(latent_t), latent.shape[1] if latent is not None else 0,
+                                         dtype_code(out_dtype), _stream()))
     return q_latent
 
 
@@ -1389,4 +1395,43 @@ def latent_attention_plain(queries: torch.Tensor, latent: torch.Tensor, block_ta
                                                  block_table.shape[1], _ptr(token_entry), _ptr(positions), n, heads,
                                                  int(rank), width - int(rank), latent.shape[1], ctypes.c_float(scale),
                                                  _ptr(sink), _ptr(out), _stream()))
+    return out
+
+
+def latent_attention_mfma_supported(queries: torch.Tensor, latent: torch.Tensor, rank: int) -> bool:
+    """The matrix-core kernel takes these operands: bfloat16, a latent and a whole row of multiples of 16 channels (up to
+    512 and 576), pages of a multiple of 8 tokens."""
+    return (queries.dtype == torch.bfloat16 and latent.dtype == torch.bfloat16
+            and bool(library().somi_latent_attention_mfma_supported(int(rank), latent.shape[2] - int(rank), latent.shape[1])))
+
+
+LATENT_SPLIT_KEYS = 64          # a key split of the matrix-core kernel is whole tiles of this many keys
+LATENT_MAX_SPLITS = 64
+
+
+def latent_attention_mfma(queries: torch.Tensor, latent: torch.Tensor, latent_t: torch.Tensor, block_table: torch.Tensor,
+                          token_entry: torch.Tensor, positions: torch.Tensor, rank: int, scale: float, sink: torch.Tensor,
+                          max_context: int) -> torch.Tensor:
+    """:func:`latent_attention_plain` on the matrix cores (bfloat16).  ``latent_t``: [pages, rank, page], the latents
+    transposed inside their pages.  ``max_context``: the longest context of the step, known to the host; a step of few
+    tokens splits every token's keys over several workgroups, so that the device is busy."""
+    _need(queries, "query rows", torch.bfloat16)
+    n, heads, width = queries.shape
+    _need(latent, "kept latents", torch.bfloat16)
+    if latent.dim() != 3 or latent.shape[2] != width or not 0 < rank <= width:
+        raise KernelError(f"latent_attention: cache {tuple(latent.shape)} does not fit queries of {width} (rank {rank})")
+    _need(latent_t, "transposed latents", torch.bfloat16, (latent.shape[0], rank, latent.shape[1]))
+    _need(block_table, "block table", torch.int32)
+    _need(token_entry, "token entries", torch.int32, (n,))
+    _need(positions, "positions", torch.int32, (n,))
+    _need(sink, "sinks", torch.float32, (heads,))
+    groups = n * ((heads + 15) // 16)
+    tiles = max(1, (int(max_context) + LATENT_SPLIT_KEYS - 1) // LATENT_SPLIT_KEYS)
+    splits = max(1, min(LATENT_MAX_SPLITS, tiles, (2 * compute_units()) // max(groups, 1)))
+    out = torch.empty((n, heads, rank), dtype=torch.bfloat16, device=queries.device)
+    part = torch.empty((n * heads * splits * (rank + 2),), dtype=torch.float32, device=queries.device) if splits > 1 else None
+    _check(library().somi_latent_attention_mfma(_ptr(queries), _ptr(latent), _ptr(latent_t), _ptr(block_table),
+                                                block_table.shape[1], _ptr(token_entry), _ptr(positions), n, heads,
+                                                int(rank), width - int(rank), latent.shape[1], ctypes.c_float(scale),
+                                                _ptr(sink), splits, _ptr(out), _ptr(part), _stream()))
     return out

@@ -111,12 +111,19 @@ class LatentAttention(Mixer):
 
     # -------------------------------------------------------------------- cache
     def cache_spec(self) -> PagedSpec:
-        return PagedSpec((PageTensor("latent", (PAGE, self.kv_rank + self.rot_dim)),), None, self.page_size)
+        """A token's row [c | r], and c once more transposed inside its page (consecutive positions of one channel
+        adjacent: the operand layout of the weights-times-latents product on the matrix cores)."""
+        return PagedSpec((PageTensor("latent", (PAGE, self.kv_rank + self.rot_dim)),
+                          PageTensor("latent_t", (self.kv_rank, PAGE))), None, self.page_size)
 
     # ------------------------------------------------------------------ forward
-    def attend(self, queries: torch.Tensor, latent: torch.Tensor, step, view) -> torch.Tensor:
+    def attend(self, queries: torch.Tensor, latent: torch.Tensor, step, view, latent_t: torch.Tensor | None = None) -> torch.Tensor:
         """The weighted sums of the kept latents for ``queries`` [N, heads, rank + rot] (the plain part already on the
-        latent's side) -> [N, heads, rank]."""
+        latent's side) -> [N, heads, rank].  bfloat16 sizes the matrix-core kernel is built for take it (it reads the
+        transposed pages ``latent_t``); float32 and other sizes take the plain kernel."""
+        if latent_t is not None and ops.latent_attention_mfma_supported(queries, latent, self.kv_rank):
+            return ops.latent_attention_mfma(queries, latent, latent_t, view.block_table, step.token_entry, step.positions,
+                                             self.kv_rank, self.scale, self.sink, step.max_context)
         return ops.latent_attention_plain(queries, latent, view.block_table, step.token_entry, step.positions,
                                           self.kv_rank, self.scale, self.sink)
 
@@ -128,7 +135,7 @@ class LatentAttention(Mixer):
         if hasattr(x, "materialize"):
             x = x.materialize()
         view = step.paged[cache.group]
-        latent = cache.tensors["latent"]
+        latent, latent_t = cache.tensors["latent"], cache.tensors.get("latent_t")
         heads, rank, rot, dtype = self.num_heads, self.kv_rank, self.rot_dim, self.runtime.dtype
         n = x.shape[0]
         with stage(self.down.label):
@@ -137,7 +144,8 @@ class LatentAttention(Mixer):
             q_latent = ops.latent_prepare(rows, self.q_rank, rank, rot, self.q_norm, self.c_norm, self.eps, self.inv_freq,
                                           self.rot_dims, self.amplitude, step.positions,
                                           None if self.shares_cache else view.slot_mapping,
-                                          None if self.shares_cache else latent, dtype)
+                                          None if self.shares_cache else latent, dtype,
+                                          None if self.shares_cache else latent_t)
         q = self.up_q(q_latent)
         with stage("queries to the latent's side"):
             queries = torch.empty((n, heads, rank + rot), dtype=dtype, device=q.device)
@@ -146,7 +154,7 @@ class LatentAttention(Mixer):
                 ops.latent_place(q, heads, self.dim, rot, rank, self.inv_freq, self.rot_dims, self.amplitude,
                                  step.positions, queries)
         with stage("attention"):
-            mixed = self.attend(queries, latent, step, view)
+            mixed = self.attend(queries, latent, step, view, latent_t)
         with stage("values from the latent"):
             values = ops.head_linear(mixed, self.value_maps).view(n, heads * self.value_dim)
         with stage(self.out.label):

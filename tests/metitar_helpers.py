@@ -31,9 +31,9 @@ def hgrn2(heads, dim, vdim, mlp=None):
 METITAR = {
     "A": dict(block_size=16, seed=15, config=MetitarConfig(
         vocab=211, width=96, norm_eps=1e-5, embedding_scale=4.0, logit_scale=0.5, token_side_dim=8, canon_taps=3, layers=(
-            latent(4, 16, 8, 24, 32, 40, 0.2, base=5000.0, scaling=RampedScaling(4.0, 64, 16.0, 2.0), mlp=MetitarDense(80)),
+            latent(4, 16, 16, 24, 32, 40, 0.2, base=5000.0, scaling=RampedScaling(4.0, 64, 16.0, 2.0), mlp=MetitarDense(80)),
             hgrn2(3, 16, 24, MetitarExperts(experts=8, top=2, ff=32, shared_ff=48)),
-            latent(2, 24, 8, 16, 32, 24, 0.25, base=5000.0, scaling=RampedScaling(4.0, 64, 16.0, 2.0), kv_from=0,
+            latent(2, 24, 16, 16, 32, 24, 0.25, base=5000.0, scaling=RampedScaling(4.0, 64, 16.0, 2.0), kv_from=0,
                    mlp=MetitarExperts(experts=6, top=3, ff=24, shared_ff=16)),
             hgrn2(2, 32, 16, None),
         ))),

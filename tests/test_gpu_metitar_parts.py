@@ -218,23 +218,31 @@ def test_one_far_key_stands_out(dtype, far, page, decoded):
     query's own neighbourhood) is made to match the last query, up to hundreds of tokens later, much better than any
     other: the output is then that vector.  The query arrives alone (a decoded token) or as the last of a portion."""
     tokens, count = 420, (1 if decoded else 12)
-    mixer, weights, config = latent_mixer(dtype, 2, 16, 8, 16, 32, 24, 1.0, page, seed=far + 1)
+    mixer, weights, config = latent_mixer(dtype, 2, 16, 16, 16, 32, 24, 1.0, page, seed=far + 1)
     x = rounded(torch.randn(tokens, 64, generator=torch.Generator().manual_seed(far)) * 0.2, dtype)
     engine = Engine(mixer, dtype, page)
     engine.run([("a", x[:tokens - count])])
     engine.cache.reserve("a", count)
     step = build_step([StepEntry("a", [0] * count, [])], engine.cache, DEV, mixer_splits(mixer))
-    cache = engine.cache.layer_caches[0].tensors["latent"]
+    cache, cache_t = (engine.cache.layer_caches[0].tensors[name] for name in ("latent", "latent_t"))
     rows = torch.tensor(engine.cache.slots(0, "a", 0, tokens), device=DEV)
-    cache.view(-1, 40)[rows[tokens - count:]] = (torch.randn(count, 40, generator=torch.Generator().manual_seed(1)) * 0.1).to(dtype).to(DEV)
-    marked = torch.zeros(40)
+
+    def keep(position, vector):
+        """Put a vector where the layer would have kept it: the row, and the latent part transposed inside its page."""
+        slot = int(rows[position])
+        cache.view(-1, 48)[slot] = vector.to(dtype).to(DEV)
+        cache_t[slot // page, :, slot % page] = vector[:32].to(dtype).to(DEV)
+    fresh = torch.randn(count, 48, generator=torch.Generator().manual_seed(1)) * 0.1
+    for i in range(count):
+        keep(tokens - count + i, fresh[i])
+    marked = torch.zeros(48)
     marked[5], marked[20] = 6.0, -3.0
-    cache.view(-1, 40)[rows[far]] = marked.to(dtype).to(DEV)
-    queries = torch.zeros(count, 2, 40)
+    keep(far, marked)
+    queries = torch.zeros(count, 2, 48)
     queries[:, :, 5] = 8.0                                   # the query's part on the latent's side points along channel 5
     queries[:, 1, 33] = 0.5
-    got = mixer.attend(queries.to(dtype).to(DEV), cache, step, step.paged[0]).float().cpu()
-    kept = cache.view(-1, 40)[rows].float().cpu()
+    got = mixer.attend(queries.to(dtype).to(DEV), cache, step, step.paged[0], cache_t).float().cpu()
+    kept = cache.view(-1, 48)[rows].float().cpu()
     scores = torch.einsum("hr,tr->ht", queries[0], kept)
     share = torch.softmax(torch.cat([scores, weights["m.sink"][:, None]], dim=1), dim=1)
     assert float(share[:, far].min()) > 0.9, "the marked key does not stand out in this test's own arithmetic"

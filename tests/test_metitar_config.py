@@ -47,7 +47,7 @@ def test_config_errors_name_the_key():
         (lambda r: r["layers"][0].__setitem__("type", "attention"), "'type'"),
         (lambda r: r["layers"][0]["mixer"].pop("kv_rank"), "kv_rank"),
         (lambda r: r["layers"][0]["mixer"]["rot"].__setitem__("dims", 7), "rot.dims"),
-        (lambda r: r["layers"][0]["mixer"]["rot"].__setitem__("dims", 10), "rot.dims"),
+        (lambda r: r["layers"][0]["mixer"]["rot"].__setitem__("dims", 18), "rot.dims"),
         (lambda r: r["layers"][2]["mixer"].__setitem__("kv_from", 1), "kv_from"),
         (lambda r: r["layers"][2]["mixer"].__setitem__("kv_from", 2), "kv_from"),
         (lambda r: r["layers"][2]["mixer"].__setitem__("kv_rank", 16), "kv_rank"),
@@ -71,15 +71,15 @@ def test_plan_names_tensors_and_borrowed_caches():
             "l2.mlp.shared.down", "l3.side.norm"} <= set(names)
     assert "l2.mix.dkv" not in names and "l2.mix.dkv.norm" not in names       # the borrower projects no latent
     assert "l3.norm2" not in names and "l3.mlp.up" not in names               # a layer without a feed-forward
-    assert names["l0.mix.uq"].shape == (4 * (16 + 8), 40) and names["l0.mix.dkv"].shape == (32 + 8, 96)
+    assert names["l0.mix.uq"].shape == (4 * (16 + 16), 40) and names["l0.mix.dkv"].shape == (32 + 16, 96)
     assert names["l2.mix.uk"].shape == (2 * 24, 32) and names["l0.canon1"].shape == (96, 3)
     assert names["side.embed"].shape == (211, 4 * 8) and not any(name.endswith(".weight") for name in names)
     model = DecoderModel(plan, Runtime(torch.float32, torch.device("cpu")))
     needs = model.cache_needs()
     assert all(isinstance(need, CompositeSpec) for need in needs)
     own, borrowed = dict(needs[0].parts), dict(needs[2].parts)
-    assert isinstance(own["mixer"], PagedSpec) and [t.name for t in own["mixer"].tensors] == ["latent"]
-    assert own["mixer"].tensors[0].elements_per_token() == 32 + 8 and own["mixer"].window is None
+    assert isinstance(own["mixer"], PagedSpec) and [t.name for t in own["mixer"].tensors] == ["latent", "latent_t"]
+    assert [t.elements_per_token() for t in own["mixer"].tensors] == [32 + 16, 32] and own["mixer"].window is None
     assert own["input"] == FixedStateSpec((2, 96), torch.float32)
     assert borrowed["mixer"] == BorrowedCache(0, ("mixer",)) and isinstance(borrowed["input"], FixedStateSpec)
     assert dict(needs[1].parts)["mixer"] == FixedStateSpec((3, 16, 24), torch.float32)
