@@ -4,8 +4,58 @@
 //     out[t, h, :] = W[h] x[t, h, :],        W: [heads, n_out, K],   x[t, h, :] at x + t * x_row + h * x_head
 //
 // The plain kernel: a workgroup owns 16 rows x 64 outputs of one head, x and W tiles go through LDS 32 channels at a
-// time, float32 sums in one order per output.
+// time, float32 sums in one order per output.  The matrix-core kernel (bfloat16, K and the strides multiples of 8,
+// outputs a multiple of 16): a workgroup owns 64 rows x 64 outputs of one head, a wavefront 16 of the rows; out^T = W x^T
+// by `16x16x32` products whose fragments come straight from memory (16 bytes a lane, K contiguous in both operands), so
+// a lane ends with 4 consecutive outputs of one row.
 #include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 hl_bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 hl_bf16x4;
+typedef __attribute__((ext_vector_type(4))) float hl_f32x4;
+#define HLM_ROWS 64
+#define HLM_TILES 4               // 16-output tiles of a workgroup
+
+__global__ void __launch_bounds__(256)
+head_linear_mfma_kernel(const bf16* __restrict__ x, int64_t x_row, int64_t x_head, const bf16* __restrict__ w, int n_rows,
+                        int n_out, int K, bf16* __restrict__ out, int64_t out_row, int64_t out_head) {
+    const int h = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = lane & 15, quad = lane >> 4;
+    const int row = blockIdx.x * HLM_ROWS + wave * 16 + col;
+    const int out0 = blockIdx.y * (HLM_TILES * 16);
+    const bf16* xr = x + (int64_t)min(row, n_rows - 1) * x_row + h * x_head;
+    const bf16* wh = w + (int64_t)h * n_out * K;
+    hl_f32x4 acc[HLM_TILES];
+#pragma unroll
+    for (int j = 0; j < HLM_TILES; ++j) acc[j] = hl_f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        const int k = k0 + quad * 8;
+        hl_bf16x8 xf, wf[HLM_TILES];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xf[i] = (__bf16)0.f;
+        if (k < K) xf = *reinterpret_cast<const hl_bf16x8*>(xr + k);
+#pragma unroll
+        for (int j = 0; j < HLM_TILES; ++j) {
+            const int o = out0 + j * 16 + col;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) wf[j][i] = (__bf16)0.f;
+            if (k < K && o < n_out) wf[j] = *reinterpret_cast<const hl_bf16x8*>(wh + (int64_t)o * K + k);
+        }
+#pragma unroll
+        for (int j = 0; j < HLM_TILES; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], xf, acc[j], 0, 0, 0);
+    }
+    if (row >= n_rows) return;
+#pragma unroll
+    for (int j = 0; j < HLM_TILES; ++j) {
+        const int o = out0 + j * 16 + quad * 4;
+        if (o >= n_out) continue;
+        hl_bf16x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = (__bf16)acc[j][i];
+        *reinterpret_cast<hl_bf16x4*>(out + (int64_t)row * out_row + h * out_head + o) = v;
+    }
+}
 
 #define HL_ROWS 16
 #define HL_COLS 64
@@ -55,6 +105,14 @@ extern "C" int somi_head_linear(const void* x, int64_t x_row, int64_t x_head, co
     SOMI_REQUIRE(n_rows >= 0 && heads > 0 && n_out > 0 && K > 0, "head_linear: bad sizes");
     SOMI_REQUIRE(heads <= 65535 && ceil_div(n_out, HL_COLS) <= 65535, "head_linear: too many heads or columns");
     if (n_rows == 0) return 0;
+    if (dtype == SOMI_BF16 && K % 8 == 0 && n_out % 16 == 0 && x_row % 8 == 0 && x_head % 8 == 0 && out_row % 4 == 0
+        && out_head % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 8 == 0) {
+        const dim3 tiles(ceil_div(n_rows, HLM_ROWS), ceil_div(n_out, HLM_TILES * 16), heads);
+        hipLaunchKernelGGL(head_linear_mfma_kernel, tiles, dim3(256), 0, stream, (const bf16*)x, x_row, x_head,
+                           (const bf16*)w, n_rows, n_out, K, (bf16*)out, out_row, out_head);
+        SOMI_LAUNCH_CHECK("head_linear_mfma");
+        return 0;
+    }
     const dim3 grid(ceil_div(n_rows, HL_ROWS), ceil_div(n_out, HL_COLS), heads);
     if (dtype == SOMI_F32)
         hipLaunchKernelGGL(head_linear_plain_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, x_row, x_head,

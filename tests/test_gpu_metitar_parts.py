@@ -377,12 +377,14 @@ def test_sigmoid_scored_experts_weigh_their_inputs(dtype, experts, top, ff, shar
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,n_out,k,rows", [(3, 32, 16, 5), (1, 7, 9, 1), (6, 96, 32, 130), (2, 160, 64, 33)])
-def test_per_head_products(dtype, heads, n_out, k, rows):
+@pytest.mark.parametrize("pads", [(5, 3), (8, 4)])          # strides the matrix-core kernel refuses, and ones it takes
+@pytest.mark.parametrize("heads,n_out,k,rows", [(3, 32, 16, 5), (1, 7, 9, 1), (6, 96, 32, 130), (2, 160, 64, 33), (16, 512, 128, 70),
+                                                (4, 48, 104, 64)])
+def test_per_head_products(dtype, pads, heads, n_out, k, rows):
     gen = torch.Generator().manual_seed(rows)
-    x = rounded(torch.randn(rows, heads, k + 5, generator=gen), dtype)
+    x = rounded(torch.randn(rows, heads, k + pads[0], generator=gen), dtype)
     w = rounded(torch.randn(heads, n_out, k, generator=gen), dtype)
-    out = torch.zeros(rows, heads, n_out + 3, dtype=dtype, device=DEV)
+    out = torch.zeros(rows, heads, n_out + pads[1], dtype=dtype, device=DEV)
     ops.head_linear(x.to(dtype).to(DEV)[:, :, :k], w.to(dtype).to(DEV), out=out[:, :, :n_out])
     want = torch.einsum("thk,hok->tho", x[:, :, :k], w)
     check(out[:, :, :n_out].float().cpu(), want, dtype, 8)
