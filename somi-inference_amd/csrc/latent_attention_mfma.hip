@@ -6,14 +6,16 @@
 // see the same keys, over one part of the token's keys (a key split); its four wavefronts walk 64-key tiles:
 //
 //   scores   wavefront w owns keys 16 w .. 16 w + 15 of the tile: S^T = K Q^T by `16x16x32` products over the rank + rot
-//            channels, K fragments straight from the rows (16 bytes a lane), the slots' Q fragments held in registers
-//            for the whole walk; a lane then holds 4 keys of one slot
+//            channels, K fragments straight from the rows (16 bytes a lane), the slots' Q fragments from LDS, where they
+//            stay for the whole walk; a lane then holds 4 keys of one slot
 //   softmax  float32, online: the running maximum of a slot starts at the head's sink and its running sum at 1 (the
 //            sink's own term, in the first key split only), the tile's maximum is exchanged through LDS
 //   values   the weights go to LDS as two bfloat16 halves (p = hi + lo, so no weight is rounded to eight bits) and
 //            come back as B operands; wavefront w owns the channel tiles w, w + 4, ... of the output, O^T = C^T P^T with
 //            the C^T fragments straight from the transposed pages
 //
+// The loads run ahead of their use: a tile's transposed latents are asked for a whole tile earlier (two sets of
+// registers), the next tile's K fragments as soon as this tile's score products have read the registers they go to.
 // A token's key splits leave (maximum, sum, unnormed output) in a workspace and a second kernel joins them.
 #include "common.h"
 
@@ -22,6 +24,13 @@ typedef __attribute__((ext_vector_type(4))) __bf16 lam_bf16x4;
 typedef __attribute__((ext_vector_type(4))) float lam_f32x4;
 
 #define LAM_KEYS 64
+
+// A barrier for data that went through LDS: waits for this wavefront's LDS traffic only, so that loads from memory
+// that were asked for ahead of their use stay in flight across it (the language's barrier waits for those as well).
+__device__ __forceinline__ void lam_lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+}
 
 template <int STEPS, int CT>
 __global__ void __launch_bounds__(256)
@@ -34,6 +43,7 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
     __shared__ float wsum[4][16];
     __shared__ __attribute__((aligned(16))) bf16 p_hi[16][LAM_KEYS + 8];
     __shared__ __attribute__((aligned(16))) bf16 p_lo[16][LAM_KEYS + 8];
+    __shared__ __attribute__((aligned(16))) bf16 q_s[16][STEPS * 32 + 8];
     const int t = n_tokens - 1 - (int)blockIdx.x;               // the longest walks first
     const int hg = blockIdx.y, split = blockIdx.z;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -49,54 +59,60 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
     const int k_begin = split * per * LAM_KEYS;
     const int k_end = min(p + 1, (split + 1) * per * LAM_KEYS);
 
-    lam_bf16x8 qf[STEPS];
+    // the slots' queries go to LDS once (rows padded by 16 bytes, so that the 16 rows of a fragment fall on different
+    // banks): held in registers they would leave no room for loads that run ahead
+    for (int i = threadIdx.x; i < 16 * STEPS * 4; i += 256) {
+        const int slot = i / (STEPS * 4), ch = (i % (STEPS * 4)) * 8;
+        lam_bf16x8 v;
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-        const int ch = s * 32 + quad * 8;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) qf[s][i] = (__bf16)0.f;
-        if (s < steps && live && ch < D)
-            qf[s] = *reinterpret_cast<const lam_bf16x8*>(queries + ((int64_t)t * heads + head) * D + ch);
+        for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.f;
+        if (hg * 16 + slot < heads && ch < D)
+            v = *reinterpret_cast<const lam_bf16x8*>(queries + ((int64_t)t * heads + hg * 16 + slot) * D + ch);
+        *reinterpret_cast<lam_bf16x8*>(&q_s[slot][ch]) = v;
     }
+    __syncthreads();
     lam_f32x4 acc[CT];
 #pragma unroll
     for (int j = 0; j < CT; ++j) acc[j] = lam_f32x4{0.f, 0.f, 0.f, 0.f};
     float m = split == 0 ? (live ? sink[head] : 0.f) : -INFINITY;
     float lsum = (split == 0 && w == 0 && quad == 0) ? 1.f : 0.f;
 
-    for (int kb = k_begin; kb < k_end; kb += LAM_KEYS) {
-        // ---- scores of this wavefront's 16 keys
+    // A tile's K fragments (this wavefront's 16 keys) and the transposed latents of the channel tiles it owns, as they
+    // are stored: nothing touches them until the products that read them.
+    auto load_keys = [&](int kb, lam_bf16x8 (&kf)[STEPS]) {
         const int key_row = min(kb + 16 * w + col, p);
         const bf16* krow = latent + ((int64_t)table[key_row / page_size] * page_size + key_row % page_size) * D;
-        lam_bf16x8 kf[STEPS];
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
             const int ch = s * 32 + quad * 8;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) kf[s][i] = (__bf16)0.f;
             if (s < steps && ch < D) kf[s] = *reinterpret_cast<const lam_bf16x8*>(krow + ch);
         }
-        lam_f32x4 sc = lam_f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < STEPS; ++s)
-            if (s < steps) sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[s], qf[s], sc, 0, 0, 0);
-        // ---- the transposed latents of the channel tiles this wavefront owns, asked for before the softmax
-        lam_bf16x8 vf[CT][2];
+    };
+    auto load_values = [&](int kb, lam_bf16x8 (&vf)[CT][2]) {
 #pragma unroll
         for (int j = 0; j < CT; ++j) {
             const int ct = w + 4 * j;
+            if (ct >= tiles_c) continue;
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) vf[j][half][i] = (__bf16)0.f;
-                if (ct < tiles_c) {
-                    const int key8 = min(kb + half * 32 + quad * 8, p & ~7);
-                    const bf16* vrow = latent_t + (((int64_t)table[key8 / page_size] * rank + ct * 16 + col) * page_size
-                                                   + key8 % page_size);
-                    vf[j][half] = *reinterpret_cast<const lam_bf16x8*>(vrow);
-                }
+                const int key8 = min(kb + half * 32 + quad * 8, p & ~7);
+                vf[j][half] = *reinterpret_cast<const lam_bf16x8*>(
+                    latent_t + (((int64_t)table[key8 / page_size] * rank + ct * 16 + col) * page_size + key8 % page_size));
             }
         }
+    };
+    // One tile: the next tile's transposed latents are asked for first (they are used a whole tile later), the next
+    // tile's K fragments right after this tile's score products have read the registers they go to.
+    auto tile = [&](int kb, lam_bf16x8 (&kf)[STEPS], lam_bf16x8 (&vf)[CT][2], lam_bf16x8 (&vnext)[CT][2]) {
+        const bool more = kb + LAM_KEYS < k_end;
+        if (more) load_values(kb + LAM_KEYS, vnext);
+        lam_f32x4 sc = lam_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s)
+            if (s < steps)
+                sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[s], *reinterpret_cast<const lam_bf16x8*>(&q_s[col][s * 32 + quad * 8]),
+                                                             sc, 0, 0, 0);
+        if (more) load_keys(kb + LAM_KEYS, kf);
         // ---- softmax over the tile, float32
         float s4[4], mx = -INFINITY;
 #pragma unroll
@@ -108,7 +124,7 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         if (quad == 0) wmax[w][col] = mx;
-        __syncthreads();
+        lam_lds_barrier();
         const float m_new = fmaxf(fmaxf(m, fmaxf(wmax[0][col], wmax[1][col])), fmaxf(wmax[2][col], wmax[3][col]));
         const float corr = __expf(m - m_new);
         m = m_new;
@@ -128,7 +144,7 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
         for (int j = 0; j < CT; ++j)
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[j][i] *= corr;
-        __syncthreads();
+        lam_lds_barrier();
         // ---- weights times latents
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
@@ -141,6 +157,25 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
                     acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j][half], pl, acc[j], 0, 0, 0);
                 }
         }
+    };
+    lam_bf16x8 kf[STEPS], va[CT][2], vb[CT][2];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) kf[s][i] = (__bf16)0.f;        // the half step past the row's end stays zero
+#pragma unroll
+    for (int j = 0; j < CT; ++j)
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) va[j][half][i] = vb[j][half][i] = (__bf16)0.f;
+    if (k_begin < k_end) {
+        load_keys(k_begin, kf);
+        load_values(k_begin, va);
+    }
+    for (int kb = k_begin; kb < k_end; kb += 2 * LAM_KEYS) {
+        tile(kb, kf, va, vb);
+        if (kb + LAM_KEYS < k_end) tile(kb + LAM_KEYS, kf, vb, va);
     }
     // ---- the slots' sums: the lane groups of a wavefront, then the wavefronts
     lsum += __shfl_xor(lsum, 16, 64);
@@ -177,20 +212,28 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
 }
 
 // out[t, h, :] = sum_s exp(m_s - M) O_s / sum_s exp(m_s - M) l_s over a token's key splits (a split without keys has
-// m = -inf and weighs nothing).  One workgroup per (token, head).
+// m = -inf and weighs nothing).  One workgroup per (token, head): the splits' weights go to LDS first, then a thread sums
+// its channels over the splits, neighbouring threads reading neighbouring channels.
+#define LAM_MAX_SPLITS 64
 __global__ void __launch_bounds__(128)
 latent_attention_join_kernel(const float* __restrict__ part, int splits, int rank, bf16* __restrict__ out) {
+    __shared__ float weight[LAM_MAX_SPLITS];
+    __shared__ float red[16];
     const int64_t slot = blockIdx.x;
     const float* mine = part + slot * splits * (rank + 2);
-    float top = -INFINITY;
-    for (int s = 0; s < splits; ++s) top = fmaxf(top, mine[s * (rank + 2) + rank]);
-    float total = 0.f;
-    for (int s = 0; s < splits; ++s) total += __expf(mine[s * (rank + 2) + rank] - top) * mine[s * (rank + 2) + rank + 1];
-    const float inv = 1.0f / total;
+    const int s_mine = threadIdx.x;
+    const float m_s = s_mine < splits ? mine[s_mine * (rank + 2) + rank] : -INFINITY;
+    const float l_s = s_mine < splits ? mine[s_mine * (rank + 2) + rank + 1] : 0.f;
+    const float top = block_max<128>(m_s, red);
+    const float e = __expf(m_s - top);
+    const float total = block_sum<128>(e * l_s, red);
+    if (s_mine < splits) weight[s_mine] = e / total;
+    __syncthreads();
     for (int c = threadIdx.x; c < rank; c += 128) {
         float sum = 0.f;
-        for (int s = 0; s < splits; ++s) sum += __expf(mine[s * (rank + 2) + rank] - top) * mine[s * (rank + 2) + c];
-        out[slot * rank + c] = (bf16)(sum * inv);
+#pragma unroll 8
+        for (int s = 0; s < splits; ++s) sum = fmaf(weight[s], mine[s * (rank + 2) + c], sum);
+        out[slot * rank + c] = (bf16)sum;
     }
 }
 
@@ -212,7 +255,7 @@ extern "C" int somi_latent_attention_mfma(const void* queries, const void* laten
                  "latent_attention_mfma: a latent of %d + %d in pages of %d is not what the kernel is built for", rank, rot,
                  page_size);
     SOMI_REQUIRE(splits == 1 || part != nullptr, "latent_attention_mfma: key splits need a workspace");
-    SOMI_REQUIRE(ceil_div(heads, 16) <= 65535 && splits <= 65535, "latent_attention_mfma: too many heads or splits");
+    SOMI_REQUIRE(ceil_div(heads, 16) <= 65535 && splits <= LAM_MAX_SPLITS, "latent_attention_mfma: too many heads or splits");
     if (n_tokens == 0) return 0;
     const int D = rank + rot;
     const dim3 grid(n_tokens, ceil_div(heads, 16), splits);
