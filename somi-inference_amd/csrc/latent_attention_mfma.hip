@@ -1,7 +1,7 @@
 // Attention over kept latents on the matrix cores (bfloat16).
 //
 // Every past token keeps one row [c (rank) | r (rot)] for all heads, and the same c once more transposed inside its
-// page ([pages, rank, page]: consecutive positions of one channel are adjacent, the operand layout of the
+// page (pages of a power of two of tokens; [pages, rank, page]: consecutive positions of one channel are adjacent, the operand layout of the
 // weights-times-values product).  A workgroup serves ONE token and up to 16 of its heads (its query slots), which all
 // see the same keys, over one part of the token's keys (a key split); its four wavefronts walk 64-key tiles:
 //
@@ -37,8 +37,9 @@ __global__ void __launch_bounds__(256)
 latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __restrict__ latent,
                              const bf16* __restrict__ latent_t, const int* __restrict__ block_table, int max_blocks,
                              const int* __restrict__ token_entry, const int* __restrict__ positions, int n_tokens,
-                             int heads, int rank, int D, int page_size, float scale, const float* __restrict__ sink,
+                             int heads, int rank, int D, int page_shift, float scale, const float* __restrict__ sink,
                              int splits, bf16* __restrict__ out, float* __restrict__ part) {
+    const int page_mask = (1 << page_shift) - 1;
     __shared__ float wmax[4][16];
     __shared__ float wsum[4][16];
     __shared__ __attribute__((aligned(16))) bf16 p_hi[16][LAM_KEYS + 8];
@@ -81,7 +82,7 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
     // are stored: nothing touches them until the products that read them.
     auto load_keys = [&](int kb, lam_bf16x8 (&kf)[STEPS]) {
         const int key_row = min(kb + 16 * w + col, p);
-        const bf16* krow = latent + ((int64_t)table[key_row / page_size] * page_size + key_row % page_size) * D;
+        const bf16* krow = latent + ((((int64_t)table[key_row >> page_shift]) << page_shift) + (key_row & page_mask)) * D;
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
             const int ch = s * 32 + quad * 8;
@@ -90,14 +91,14 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
     };
     auto load_values = [&](int kb, lam_bf16x8 (&vf)[CT][2]) {
 #pragma unroll
-        for (int j = 0; j < CT; ++j) {
-            const int ct = w + 4 * j;
-            if (ct >= tiles_c) continue;
+        for (int half = 0; half < 2; ++half) {
+            // the lane's 8 keys lie in one page: its channel rows there, one page lookup for all channel tiles
+            const int key8 = min(kb + half * 32 + quad * 8, p & ~7);
+            const bf16* rows = latent_t + ((((int64_t)table[key8 >> page_shift] * rank + col) << page_shift) + (key8 & page_mask));
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const int key8 = min(kb + half * 32 + quad * 8, p & ~7);
-                vf[j][half] = *reinterpret_cast<const lam_bf16x8*>(
-                    latent_t + (((int64_t)table[key8 / page_size] * rank + ct * 16 + col) * page_size + key8 % page_size));
+            for (int j = 0; j < CT; ++j) {
+                const int ct = w + 4 * j;
+                if (ct < tiles_c) vf[j][half] = *reinterpret_cast<const lam_bf16x8*>(rows + ((int64_t)(ct * 16) << page_shift));
             }
         }
     };
@@ -107,11 +108,13 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
         const bool more = kb + LAM_KEYS < k_end;
         if (more) load_values(kb + LAM_KEYS, vnext);
         lam_f32x4 sc = lam_f32x4{0.f, 0.f, 0.f, 0.f};
+        int q_at = col * (STEPS * 32 + 8) + quad * 8;        // opaque once a tile: the Q fragments are read at every use
+        asm volatile("" : "+v"(q_at));
+        const bf16* q_lane = &q_s[0][0] + q_at;
 #pragma unroll
         for (int s = 0; s < STEPS; ++s)
             if (s < steps)
-                sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[s], *reinterpret_cast<const lam_bf16x8*>(&q_s[col][s * 32 + quad * 8]),
-                                                             sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[s], *reinterpret_cast<const lam_bf16x8*>(q_lane + s * 32), sc, 0, 0, 0);
         if (more) load_keys(kb + LAM_KEYS, kf);
         // ---- softmax over the tile, float32
         float s4[4], mx = -INFINITY;
@@ -140,10 +143,12 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
         lsum = lsum * corr + psum;
         *reinterpret_cast<lam_bf16x4*>(&p_hi[col][16 * w + quad * 4]) = hi;
         *reinterpret_cast<lam_bf16x4*>(&p_lo[col][16 * w + quad * 4]) = lo;
+        if (__any(corr != 1.0f)) {                               // only where some slot's maximum moved
 #pragma unroll
-        for (int j = 0; j < CT; ++j)
+            for (int j = 0; j < CT; ++j)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[j][i] *= corr;
+                for (int i = 0; i < 4; ++i) acc[j][i] *= corr;
+        }
         lam_lds_barrier();
         // ---- weights times latents
 #pragma unroll
@@ -211,6 +216,219 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
     }
 }
 
+// The same for prompt portions: a workgroup serves LAM_TT consecutive tokens of the step (and up to 16 heads of each:
+// 16 LAM_TT query slots), so that a tile of kept rows is read once for all of them.  Tokens of one request stand side
+// by side with rising positions; where a group of tokens holds several requests (a portion's end beside the next
+// entry) the workgroup takes them run by run.  A wavefront again owns 16 keys of a tile for the scores (one K fragment
+// against the LAM_TT tokens' Q fragments from LDS) and a quarter of the channel tiles for the output (every token's).
+// The transposed latents of a tile are asked for before its scores, the next tile's K fragments after them.
+#define LAM_TT 4
+#define LAM_PW 8                      // wavefronts of a workgroup of the portion kernel
+#define LAM_PKEYS (16 * LAM_PW)       // keys of its tiles
+
+template <int STEPS, int CT>
+__global__ void __launch_bounds__(64 * LAM_PW)
+latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __restrict__ latent,
+                                const bf16* __restrict__ latent_t, const int* __restrict__ block_table, int max_blocks,
+                                const int* __restrict__ token_entry, const int* __restrict__ positions, int n_tokens,
+                                int heads, int rank, int D, int page_shift, float scale, const float* __restrict__ sink,
+                                bf16* __restrict__ out) {
+    const int page_mask = (1 << page_shift) - 1;
+    constexpr int SLOTS = 16 * LAM_TT, QROW = STEPS * 32 + 8, PROW = LAM_PKEYS + 8, NT = 64 * LAM_PW;
+    extern __shared__ __attribute__((aligned(16))) char lam_lds[];
+    bf16 (*q_s)[QROW] = reinterpret_cast<bf16 (*)[QROW]>(lam_lds);
+    bf16 (*p_hi)[PROW] = reinterpret_cast<bf16 (*)[PROW]>(lam_lds + (size_t)SLOTS * QROW * 2);
+    bf16 (*p_lo)[PROW] = reinterpret_cast<bf16 (*)[PROW]>(lam_lds + (size_t)SLOTS * QROW * 2 + (size_t)SLOTS * PROW * 2);
+    float (*wmax)[SLOTS] = reinterpret_cast<float (*)[SLOTS]>(lam_lds + (size_t)SLOTS * QROW * 2 + (size_t)SLOTS * PROW * 4);
+    const int groups = (n_tokens + LAM_TT - 1) / LAM_TT;
+    const int t0 = (groups - 1 - (int)blockIdx.x) * LAM_TT;      // the longest walks first
+    const int count = min(LAM_TT, n_tokens - t0);
+    const int hg = blockIdx.y;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int col = lane & 15, quad = lane >> 4;
+    const int head = hg * 16 + col;
+    const int steps = (D + 31) >> 5, tiles_c = rank >> 4;
+
+    for (int r0 = 0; r0 < count;) {
+        const int entry = token_entry[t0 + r0];
+        int r1 = r0 + 1;
+        while (r1 < count && token_entry[t0 + r1] == entry) ++r1;
+        const int* table = block_table + (int64_t)entry * max_blocks;
+        const int p_last = positions[t0 + r1 - 1];
+        int pos[LAM_TT];
+        bool live[LAM_TT];
+#pragma unroll
+        for (int u = 0; u < LAM_TT; ++u) {
+            live[u] = u >= r0 && u < r1;
+            pos[u] = live[u] ? positions[t0 + u] : -1;
+        }
+        for (int i = threadIdx.x; i < SLOTS * STEPS * 4; i += NT) {
+            const int slot = i / (STEPS * 4), ch = (i % (STEPS * 4)) * 8;
+            const int u = slot >> 4, h = hg * 16 + (slot & 15);
+            lam_bf16x8 v;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.f;
+            if (u >= r0 && u < r1 && h < heads && ch < D)
+                v = *reinterpret_cast<const lam_bf16x8*>(queries + ((int64_t)(t0 + u) * heads + h) * D + ch);
+            *reinterpret_cast<lam_bf16x8*>(&q_s[slot][ch]) = v;
+        }
+        __syncthreads();
+        lam_f32x4 acc[LAM_TT][CT];
+        float m[LAM_TT], lsum[LAM_TT];
+#pragma unroll
+        for (int u = 0; u < LAM_TT; ++u) {
+#pragma unroll
+            for (int j = 0; j < CT; ++j) acc[u][j] = lam_f32x4{0.f, 0.f, 0.f, 0.f};
+            m[u] = live[u] && head < heads ? sink[head] : 0.f;
+            lsum[u] = (live[u] && w == 0 && quad == 0) ? 1.f : 0.f;
+        }
+        lam_bf16x8 kf[STEPS], vf[CT][2];
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) kf[s][i] = (__bf16)0.f;        // the half step past the row's end stays zero
+        auto load_keys = [&](int kb) {
+            const int key_row = min(kb + 16 * w + col, p_last);
+            const bf16* krow = latent + ((((int64_t)table[key_row >> page_shift]) << page_shift) + (key_row & page_mask)) * D;
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) {
+                const int ch = s * 32 + quad * 8;
+                if (s < steps && ch < D) kf[s] = *reinterpret_cast<const lam_bf16x8*>(krow + ch);
+            }
+        };
+        // the transposed latents of two 32-key steps of a tile at a time (a tile has LAM_PW / 2 of them)
+        auto load_values = [&](int kb, int pair) {
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                // the lane's 8 keys lie in one page: its channel rows there, one page lookup for all channel tiles
+                const int key8 = min(kb + (2 * pair + half) * 32 + quad * 8, p_last & ~7);
+                const bf16* rows = latent_t + ((((int64_t)table[key8 >> page_shift] * rank + col) << page_shift) + (key8 & page_mask));
+#pragma unroll
+                for (int j = 0; j < CT; ++j) {
+                    const int ct = w + LAM_PW * j;
+                    if (ct < tiles_c) vf[j][half] = *reinterpret_cast<const lam_bf16x8*>(rows + ((int64_t)(ct * 16) << page_shift));
+                }
+            }
+        };
+        load_keys(0);
+        for (int kb = 0; kb <= p_last; kb += LAM_PKEYS) {
+            load_values(kb, 0);
+            lam_f32x4 sc[LAM_TT];
+#pragma unroll
+            for (int u = 0; u < LAM_TT; ++u) sc[u] = lam_f32x4{0.f, 0.f, 0.f, 0.f};
+            // the offset of the lane's Q fragments is made opaque once a tile: the fragments are read from LDS at every
+            // use instead of being kept in registers across the walk, which they would fill
+            int q_at = col * QROW + quad * 8;
+            asm volatile("" : "+v"(q_at));
+            const bf16* q_lane = &q_s[0][0] + q_at;
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+                if (s < steps) {
+#pragma unroll
+                    for (int u = 0; u < LAM_TT; ++u)
+                        if (live[u])
+                            sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                                kf[s], *reinterpret_cast<const lam_bf16x8*>(q_lane + u * 16 * QROW + s * 32), sc[u], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);       // a step's Q fragments are read when the step comes, not ahead
+                }
+            if (kb + LAM_PKEYS <= p_last) load_keys(kb + LAM_PKEYS);
+            // ---- softmax over the tile, float32, slot by slot
+            float s4[LAM_TT][4];
+#pragma unroll
+            for (int u = 0; u < LAM_TT; ++u) {
+                float mx = -INFINITY;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = kb + 16 * w + quad * 4 + i;
+                    s4[u][i] = key <= pos[u] ? sc[u][i] * scale : -INFINITY;
+                    mx = fmaxf(mx, s4[u][i]);
+                }
+                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                if (quad == 0) wmax[w][u * 16 + col] = mx;
+            }
+            lam_lds_barrier();
+#pragma unroll
+            for (int u = 0; u < LAM_TT; ++u) {
+                const int slot = u * 16 + col;
+                float m_new = m[u];
+#pragma unroll
+                for (int x = 0; x < LAM_PW; ++x) m_new = fmaxf(m_new, wmax[x][slot]);
+                const float corr = __expf(m[u] - m_new);
+                m[u] = m_new;
+                float psum = 0.f;
+                lam_bf16x4 hi, lo;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float pv = __expf(s4[u][i] - m_new);          // exp(-inf) = 0 for keys that are not seen
+                    psum += pv;
+                    hi[i] = (__bf16)pv;
+                    lo[i] = (__bf16)(pv - (float)hi[i]);
+                }
+                lsum[u] = lsum[u] * corr + psum;
+                *reinterpret_cast<lam_bf16x4*>(&p_hi[slot][16 * w + quad * 4]) = hi;
+                *reinterpret_cast<lam_bf16x4*>(&p_lo[slot][16 * w + quad * 4]) = lo;
+#pragma unroll
+                for (int j = 0; j < CT; ++j)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[u][j][i] *= corr;
+            }
+            lam_lds_barrier();
+            // ---- weights times latents, two 32-key steps at a time; the next two are asked for as soon as these have
+            //      been read
+#pragma unroll
+            for (int pair = 0; pair < LAM_PW / 4; ++pair) {
+#pragma unroll
+                for (int half = 0; half < 2; ++half)
+#pragma unroll
+                    for (int u = 0; u < LAM_TT; ++u) {
+                        if (!live[u]) continue;
+                        const int at = (2 * pair + half) * 32 + quad * 8;
+                        const lam_bf16x8 ph = *reinterpret_cast<const lam_bf16x8*>(&p_hi[u * 16 + col][at]);
+                        const lam_bf16x8 pl = *reinterpret_cast<const lam_bf16x8*>(&p_lo[u * 16 + col][at]);
+#pragma unroll
+                        for (int j = 0; j < CT; ++j)
+                            if (w + LAM_PW * j < tiles_c) {
+                                acc[u][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j][half], ph, acc[u][j], 0, 0, 0);
+                                acc[u][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j][half], pl, acc[u][j], 0, 0, 0);
+                            }
+                    }
+                if (pair + 1 < LAM_PW / 4) load_values(kb, pair + 1);
+            }
+        }
+        // ---- the slots' sums (the lane groups of a wavefront, then the wavefronts; wmax is free again) and the output
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < LAM_TT; ++u) {
+            float v = lsum[u];
+            v += __shfl_xor(v, 16, 64);
+            v += __shfl_xor(v, 32, 64);
+            if (quad == 0) wmax[w][u * 16 + col] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < LAM_TT; ++u) {
+            if (!live[u] || head >= heads) continue;
+            const int slot = u * 16 + col;
+            float total = 0.f;
+#pragma unroll
+            for (int x = 0; x < LAM_PW; ++x) total += wmax[x][slot];
+            const float inv = 1.0f / total;
+#pragma unroll
+            for (int j = 0; j < CT; ++j) {
+                const int ct = w + LAM_PW * j;
+                if (ct >= tiles_c) continue;
+                lam_bf16x4 o;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[i] = (__bf16)(acc[u][j][i] * inv);
+                *reinterpret_cast<lam_bf16x4*>(out + ((int64_t)(t0 + u) * heads + head) * rank + ct * 16 + quad * 4) = o;
+            }
+        }
+        __syncthreads();
+        r0 = r1;
+    }
+}
+
 // out[t, h, :] = sum_s exp(m_s - M) O_s / sum_s exp(m_s - M) l_s over a token's key splits (a split without keys has
 // m = -inf and weighs nothing).  One workgroup per (token, head): the splits' weights go to LDS first, then a thread sums
 // its channels over the splits, neighbouring threads reading neighbouring channels.
@@ -239,7 +457,8 @@ latent_attention_join_kernel(const float* __restrict__ part, int splits, int ran
 
 extern "C" int somi_latent_attention_mfma_supported(int rank, int rot, int page_size) {
     const int D = rank + rot;
-    return rank > 0 && rank % 16 == 0 && D % 16 == 0 && D <= 576 && rank <= 512 && page_size % 8 == 0;
+    return rank > 0 && rank % 16 == 0 && D % 16 == 0 && D <= 576 && rank <= 512 && page_size >= 8
+           && (page_size & (page_size - 1)) == 0;
 }
 
 // queries: [n_tokens, heads, rank + rot] bfloat16; latent: [pages, page, rank + rot]; latent_t: [pages, rank, page];
@@ -248,7 +467,7 @@ extern "C" int somi_latent_attention_mfma_supported(int rank, int rot, int page_
 extern "C" int somi_latent_attention_mfma(const void* queries, const void* latent, const void* latent_t,
                                           const int* block_table, int max_blocks, const int* token_entry,
                                           const int* positions, int n_tokens, int heads, int rank, int rot, int page_size,
-                                          float scale, const float* sink, int splits, void* out, float* part,
+                                          float scale, const float* sink, int splits, int portions, void* out, float* part,
                                           hipStream_t stream) {
     SOMI_REQUIRE(n_tokens >= 0 && heads > 0 && max_blocks > 0 && splits >= 1, "latent_attention_mfma: bad sizes");
     SOMI_REQUIRE(somi_latent_attention_mfma_supported(rank, rot, page_size),
@@ -258,11 +477,34 @@ extern "C" int somi_latent_attention_mfma(const void* queries, const void* laten
     SOMI_REQUIRE(ceil_div(heads, 16) <= 65535 && splits <= LAM_MAX_SPLITS, "latent_attention_mfma: too many heads or splits");
     if (n_tokens == 0) return 0;
     const int D = rank + rot;
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+    if (portions) {
+        // prompt portions: LAM_TT tokens a workgroup, no key splits
+        SOMI_REQUIRE(splits == 1, "latent_attention_mfma: prompt portions take no key splits");
+        const dim3 groups(ceil_div(n_tokens, LAM_TT), ceil_div(heads, 16));
+#define LAM_PORTION(STEPS, CT)                                                                                          \
+    do {                                                                                                                \
+        const size_t lds = (size_t)16 * LAM_TT * ((STEPS * 32 + 8) * 2 + (LAM_PKEYS + 8) * 4 + LAM_PW * 4);             \
+        hipError_t err = hipFuncSetAttribute((const void*)latent_attention_portion_kernel<STEPS, CT>,                   \
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
+        if (err != hipSuccess) return somi_fail("latent_attention_mfma: %s", hipGetErrorString(err));                   \
+        hipLaunchKernelGGL((latent_attention_portion_kernel<STEPS, CT>), groups, dim3(64 * LAM_PW), lds, stream,                \
+                           (const bf16*)queries, (const bf16*)latent, (const bf16*)latent_t, block_table, max_blocks,  \
+                           token_entry, positions, n_tokens, heads, rank, D, page_shift, scale, sink, (bf16*)out);       \
+    } while (0)
+        if (D <= 128 && rank <= 128) LAM_PORTION(4, 1);
+        else if (D <= 256 && rank <= 256) LAM_PORTION(8, 2);
+        else LAM_PORTION(18, 4);
+#undef LAM_PORTION
+        SOMI_LAUNCH_CHECK("latent_attention_portion");
+        return 0;
+    }
     const dim3 grid(n_tokens, ceil_div(heads, 16), splits);
 #define LAM_LAUNCH(STEPS, CT)                                                                                          \
     hipLaunchKernelGGL((latent_attention_mfma_kernel<STEPS, CT>), grid, dim3(256), 0, stream, (const bf16*)queries,     \
                        (const bf16*)latent, (const bf16*)latent_t, block_table, max_blocks, token_entry, positions,    \
-                       n_tokens, heads, rank, D, page_size, scale, sink, splits, (bf16*)out, part)
+                       n_tokens, heads, rank, D, page_shift, scale, sink, splits, (bf16*)out, part)
     if (D <= 128 && rank <= 128) LAM_LAUNCH(4, 2);
     else if (D <= 256 && rank <= 256) LAM_LAUNCH(8, 4);
     else LAM_LAUNCH(18, 8);

@@ -1400,7 +1400,7 @@ def latent_attention_plain(queries: torch.Tensor, latent: torch.Tensor, block_ta
 
 def latent_attention_mfma_supported(queries: torch.Tensor, latent: torch.Tensor, rank: int) -> bool:
     """The matrix-core kernel takes these operands: bfloat16, a latent and a whole row of multiples of 16 channels (up to
-    512 and 576), pages of a multiple of 8 tokens."""
+    512 and 576), pages of a power of two of at least 8 tokens."""
     return (queries.dtype == torch.bfloat16 and latent.dtype == torch.bfloat16
             and bool(library().somi_latent_attention_mfma_supported(int(rank), latent.shape[2] - int(rank), latent.shape[1])))
 
@@ -1411,10 +1411,12 @@ LATENT_MAX_SPLITS = 64
 
 def latent_attention_mfma(queries: torch.Tensor, latent: torch.Tensor, latent_t: torch.Tensor, block_table: torch.Tensor,
                           token_entry: torch.Tensor, positions: torch.Tensor, rank: int, scale: float, sink: torch.Tensor,
-                          max_context: int) -> torch.Tensor:
+                          max_context: int, portions: bool = False) -> torch.Tensor:
     """:func:`latent_attention_plain` on the matrix cores (bfloat16).  ``latent_t``: [pages, rank, page], the latents
     transposed inside their pages.  ``max_context``: the longest context of the step, known to the host; a step of few
-    tokens splits every token's keys over several workgroups, so that the device is busy."""
+    tokens splits every token's keys over several workgroups, so that the device is busy.  ``portions``: the step holds
+    prompt portions: four consecutive tokens share a workgroup, so that it reads a tile of kept rows once for all of
+    them (tokens of other requests in such a group are taken one after another)."""
     _need(queries, "query rows", torch.bfloat16)
     n, heads, width = queries.shape
     _need(latent, "kept latents", torch.bfloat16)
@@ -1427,11 +1429,11 @@ def latent_attention_mfma(queries: torch.Tensor, latent: torch.Tensor, latent_t:
     _need(sink, "sinks", torch.float32, (heads,))
     groups = n * ((heads + 15) // 16)
     tiles = max(1, (int(max_context) + LATENT_SPLIT_KEYS - 1) // LATENT_SPLIT_KEYS)
-    splits = max(1, min(LATENT_MAX_SPLITS, tiles, (2 * compute_units()) // max(groups, 1)))
+    splits = 1 if portions else max(1, min(LATENT_MAX_SPLITS, tiles, (2 * compute_units()) // max(groups, 1)))
     out = torch.empty((n, heads, rank), dtype=torch.bfloat16, device=queries.device)
     part = torch.empty((n * heads * splits * (rank + 2),), dtype=torch.float32, device=queries.device) if splits > 1 else None
     _check(library().somi_latent_attention_mfma(_ptr(queries), _ptr(latent), _ptr(latent_t), _ptr(block_table),
                                                 block_table.shape[1], _ptr(token_entry), _ptr(positions), n, heads,
                                                 int(rank), width - int(rank), latent.shape[1], ctypes.c_float(scale),
-                                                _ptr(sink), splits, _ptr(out), _ptr(part), _stream()))
+                                                _ptr(sink), splits, 1 if portions else 0, _ptr(out), _ptr(part), _stream()))
     return out

@@ -34,6 +34,7 @@ from .registry import build_part
 
 class LatentAttention(Mixer):
     graph_safe = True
+    PORTION_TOKENS = 8     # a step whose longest entry has this many tokens runs the kernel that shares a workgroup among tokens
 
     ROLES = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv",
              "sink": "sink", "o": "o", "position": "rotary_emb"}
@@ -123,7 +124,8 @@ class LatentAttention(Mixer):
         transposed pages ``latent_t``); float32 and other sizes take the plain kernel."""
         if latent_t is not None and ops.latent_attention_mfma_supported(queries, latent, self.kv_rank):
             return ops.latent_attention_mfma(queries, latent, latent_t, view.block_table, step.token_entry, step.positions,
-                                             self.kv_rank, self.scale, self.sink, step.max_context)
+                                             self.kv_rank, self.scale, self.sink, step.max_context,
+                                             portions=step.max_entry_len >= self.PORTION_TOKENS)
         return ops.latent_attention_plain(queries, latent, view.block_table, step.token_entry, step.positions,
                                           self.kv_rank, self.scale, self.sink)
 
