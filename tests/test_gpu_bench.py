@@ -144,3 +144,27 @@ def test_rusolorn_option_runs_both_models_and_leaves_the_default_alone():
         assert "attention" in line[model]["stages"]["prefill_512"] and "recurrence" in line[model]["stages"]["prefill_512"]
     assert "experts gate_up" in line["rusolorn"]["stages"]["prefill_512"] and line["value"] == line["rusolorn"]["decode_b8"]["tok_s"]
     assert line["prefill_kernels"]["rusolorn_experts"]["ms"] > 0 and line["decode_kernels"]["rusolorn_recurrence"]["ms"] > 0
+
+
+def test_metitar_option_runs_both_models_and_leaves_the_default_alone():
+    """``--metitar`` runs a Metitar model beside the closest Rusolorn model and prints one JSON line; the sizes' config
+    dictionaries build through the registry like any config.json."""
+    sys.path.insert(0, ROOT)
+    import bench
+    from somi_inference_amd.config import config_from_dict
+    for sizes in bench.METITAR_SIZES:
+        arch, config = config_from_dict(bench.metitar_config_dict(sizes))
+        assert arch.name == "Metitar" and len(config.layers) == bench.METITAR_LAYERS and config.layers[5].mixer.kv_from == 3
+        assert [layer.type for layer in config.layers].count("hgrn2") == 3 and config.canon_taps and config.token_side_dim
+        arch, closest = config_from_dict(bench.metitar_closest_config_dict(sizes))
+        assert arch.name == "Rusolorn" and len(closest.layers) == bench.METITAR_LAYERS
+        assert closest.layers[0].mlp.ff == config.layers[1].mlp.ff and closest.width == config.width
+    done = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--metitar", "1b", "--steps", "16", "--warmup", "2",
+                           "--prefill-tokens", "512", "--context", "1024"], capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-3000:]
+    line = json.loads(done.stdout.strip().splitlines()[-1])
+    for model in ("metitar", "closest"):
+        assert line[model]["prefill"]["512"]["value"] > 0 and line[model]["decode_b8"]["tok_s"] > 0
+        assert "attention" in line[model]["stages"]["prefill_512"] and "recurrence" in line[model]["stages"]["prefill_512"]
+    assert "experts gate_up" in line["metitar"]["stages"]["prefill_512"] and line["value"] == line["metitar"]["decode_b8"]["tok_s"]
+    assert line["prefill_kernels"]["metitar_attention"]["ms"] > 0 and line["decode_kernels"]["metitar_recurrence"]["ms"] > 0
