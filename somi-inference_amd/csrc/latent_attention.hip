@@ -138,7 +138,7 @@ extern "C" int somi_latent_place(const void* q, int dtype, int n_tokens, int hea
 
 // ------------------------------------------------------------------------------------------------ plain attention
 #define LATENT_PLAIN_NT 128
-#define LATENT_PLAIN_ACC 4            // value channels a thread sums: rank <= 4 * 128
+#define LATENT_PLAIN_ACC 8            // value channels a thread sums: rank <= 8 * 128
 
 template <typename T>
 __global__ void __launch_bounds__(LATENT_PLAIN_NT)
@@ -161,7 +161,9 @@ latent_attention_plain_kernel(const T* __restrict__ queries, const T* __restrict
     for (int d = tid; d < D; d += NT) qs[d] = to_float(queries[((int64_t)t * heads + h) * D + d]);
 
     float m = sink[h], l = 1.f;                // the sink: a term exp(sink - m) with no value
-    float acc[LATENT_PLAIN_ACC] = {0.f, 0.f, 0.f, 0.f};
+    float acc[LATENT_PLAIN_ACC];
+#pragma unroll
+    for (int r = 0; r < LATENT_PLAIN_ACC; ++r) acc[r] = 0.f;
     for (int tile = 0; tile <= p / NT; ++tile) {
         const int pos = tile * NT + tid;
         const bool valid = pos <= p;

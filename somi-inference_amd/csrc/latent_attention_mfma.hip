@@ -216,33 +216,33 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
     }
 }
 
-// The same for prompt portions: a workgroup serves LAM_TT consecutive tokens of the step (and up to 16 heads of each:
-// 16 LAM_TT query slots), so that a tile of kept rows is read once for all of them.  Tokens of one request stand side
+// The same for prompt portions: a workgroup serves TT consecutive tokens of the step (and up to 16 heads of each:
+// 16 TT query slots), so that a tile of kept rows is read once for all of them.  Tokens of one request stand side
 // by side with rising positions; where a group of tokens holds several requests (a portion's end beside the next
 // entry) the workgroup takes them run by run.  A wavefront again owns 16 keys of a tile for the scores (one K fragment
-// against the LAM_TT tokens' Q fragments from LDS) and a quarter of the channel tiles for the output (every token's).
+// against the TT tokens' Q fragments from LDS) and a quarter of the channel tiles for the output (every token's).
 // The transposed latents of a tile are asked for before its scores, the next tile's K fragments after them.
-#define LAM_TT 4
-#define LAM_PW 8                      // wavefronts of a workgroup of the portion kernel
-#define LAM_PKEYS (16 * LAM_PW)       // keys of its tiles
+// TT: tokens of a workgroup; PW: its wavefronts (a tile is 16 PW keys); WPS: wavefronts a SIMD is to hold (2 = two
+// workgroups of four wavefronts a compute unit, so that one's softmax runs under the other's matrix instructions).
 
-template <int STEPS, int CT>
-__global__ void __launch_bounds__(64 * LAM_PW)
+template <int STEPS, int CT, int TT, int PW, int WPS>
+__global__ void __launch_bounds__(64 * PW, WPS)
 latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __restrict__ latent,
                                 const bf16* __restrict__ latent_t, const int* __restrict__ block_table, int max_blocks,
                                 const int* __restrict__ token_entry, const int* __restrict__ positions, int n_tokens,
                                 int heads, int rank, int D, int page_shift, float scale, const float* __restrict__ sink,
                                 bf16* __restrict__ out) {
     const int page_mask = (1 << page_shift) - 1;
-    constexpr int SLOTS = 16 * LAM_TT, QROW = STEPS * 32 + 8, PROW = LAM_PKEYS + 8, NT = 64 * LAM_PW;
+    constexpr int VH = CT >= 8 ? 1 : 2;          // 32-key steps whose transposed latents are in registers at a time
+    constexpr int SLOTS = 16 * TT, QROW = STEPS * 32 + 8, PROW = (16 * PW) + 8, NT = 64 * PW;
     extern __shared__ __attribute__((aligned(16))) char lam_lds[];
     bf16 (*q_s)[QROW] = reinterpret_cast<bf16 (*)[QROW]>(lam_lds);
     bf16 (*p_hi)[PROW] = reinterpret_cast<bf16 (*)[PROW]>(lam_lds + (size_t)SLOTS * QROW * 2);
     bf16 (*p_lo)[PROW] = reinterpret_cast<bf16 (*)[PROW]>(lam_lds + (size_t)SLOTS * QROW * 2 + (size_t)SLOTS * PROW * 2);
     float (*wmax)[SLOTS] = reinterpret_cast<float (*)[SLOTS]>(lam_lds + (size_t)SLOTS * QROW * 2 + (size_t)SLOTS * PROW * 4);
-    const int groups = (n_tokens + LAM_TT - 1) / LAM_TT;
-    const int t0 = (groups - 1 - (int)blockIdx.x) * LAM_TT;      // the longest walks first
-    const int count = min(LAM_TT, n_tokens - t0);
+    const int groups = (n_tokens + TT - 1) / TT;
+    const int t0 = (groups - 1 - (int)blockIdx.x) * TT;      // the longest walks first
+    const int count = min(TT, n_tokens - t0);
     const int hg = blockIdx.y;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int col = lane & 15, quad = lane >> 4;
@@ -255,10 +255,10 @@ latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __
         while (r1 < count && token_entry[t0 + r1] == entry) ++r1;
         const int* table = block_table + (int64_t)entry * max_blocks;
         const int p_last = positions[t0 + r1 - 1];
-        int pos[LAM_TT];
-        bool live[LAM_TT];
+        int pos[TT];
+        bool live[TT];
 #pragma unroll
-        for (int u = 0; u < LAM_TT; ++u) {
+        for (int u = 0; u < TT; ++u) {
             live[u] = u >= r0 && u < r1;
             pos[u] = live[u] ? positions[t0 + u] : -1;
         }
@@ -273,16 +273,16 @@ latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __
             *reinterpret_cast<lam_bf16x8*>(&q_s[slot][ch]) = v;
         }
         __syncthreads();
-        lam_f32x4 acc[LAM_TT][CT];
-        float m[LAM_TT], lsum[LAM_TT];
+        lam_f32x4 acc[TT][CT];
+        float m[TT], lsum[TT];
 #pragma unroll
-        for (int u = 0; u < LAM_TT; ++u) {
+        for (int u = 0; u < TT; ++u) {
 #pragma unroll
             for (int j = 0; j < CT; ++j) acc[u][j] = lam_f32x4{0.f, 0.f, 0.f, 0.f};
             m[u] = live[u] && head < heads ? sink[head] : 0.f;
             lsum[u] = (live[u] && w == 0 && quad == 0) ? 1.f : 0.f;
         }
-        lam_bf16x8 kf[STEPS], vf[CT][2];
+        lam_bf16x8 kf[STEPS], vf[CT][VH];
 #pragma unroll
         for (int s = 0; s < STEPS; ++s)
 #pragma unroll
@@ -296,26 +296,26 @@ latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __
                 if (s < steps && ch < D) kf[s] = *reinterpret_cast<const lam_bf16x8*>(krow + ch);
             }
         };
-        // the transposed latents of two 32-key steps of a tile at a time (a tile has LAM_PW / 2 of them)
+        // the transposed latents of VH 32-key steps of a tile at a time (a tile has PW / 2 of them)
         auto load_values = [&](int kb, int pair) {
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
+            for (int half = 0; half < VH; ++half) {
                 // the lane's 8 keys lie in one page: its channel rows there, one page lookup for all channel tiles
-                const int key8 = min(kb + (2 * pair + half) * 32 + quad * 8, p_last & ~7);
+                const int key8 = min(kb + (VH * pair + half) * 32 + quad * 8, p_last & ~7);
                 const bf16* rows = latent_t + ((((int64_t)table[key8 >> page_shift] * rank + col) << page_shift) + (key8 & page_mask));
 #pragma unroll
                 for (int j = 0; j < CT; ++j) {
-                    const int ct = w + LAM_PW * j;
+                    const int ct = w + PW * j;
                     if (ct < tiles_c) vf[j][half] = *reinterpret_cast<const lam_bf16x8*>(rows + ((int64_t)(ct * 16) << page_shift));
                 }
             }
         };
         load_keys(0);
-        for (int kb = 0; kb <= p_last; kb += LAM_PKEYS) {
+        for (int kb = 0; kb <= p_last; kb += (16 * PW)) {
             load_values(kb, 0);
-            lam_f32x4 sc[LAM_TT];
+            lam_f32x4 sc[TT];
 #pragma unroll
-            for (int u = 0; u < LAM_TT; ++u) sc[u] = lam_f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int u = 0; u < TT; ++u) sc[u] = lam_f32x4{0.f, 0.f, 0.f, 0.f};
             // the offset of the lane's Q fragments is made opaque once a tile: the fragments are read from LDS at every
             // use instead of being kept in registers across the walk, which they would fill
             int q_at = col * QROW + quad * 8;
@@ -325,17 +325,17 @@ latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __
             for (int s = 0; s < STEPS; ++s)
                 if (s < steps) {
 #pragma unroll
-                    for (int u = 0; u < LAM_TT; ++u)
+                    for (int u = 0; u < TT; ++u)
                         if (live[u])
                             sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                                 kf[s], *reinterpret_cast<const lam_bf16x8*>(q_lane + u * 16 * QROW + s * 32), sc[u], 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);       // a step's Q fragments are read when the step comes, not ahead
                 }
-            if (kb + LAM_PKEYS <= p_last) load_keys(kb + LAM_PKEYS);
+            if (kb + (16 * PW) <= p_last) load_keys(kb + (16 * PW));
             // ---- softmax over the tile, float32, slot by slot
-            float s4[LAM_TT][4];
+            float s4[TT][4];
 #pragma unroll
-            for (int u = 0; u < LAM_TT; ++u) {
+            for (int u = 0; u < TT; ++u) {
                 float mx = -INFINITY;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
@@ -349,11 +349,11 @@ latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __
             }
             lam_lds_barrier();
 #pragma unroll
-            for (int u = 0; u < LAM_TT; ++u) {
+            for (int u = 0; u < TT; ++u) {
                 const int slot = u * 16 + col;
                 float m_new = m[u];
 #pragma unroll
-                for (int x = 0; x < LAM_PW; ++x) m_new = fmaxf(m_new, wmax[x][slot]);
+                for (int x = 0; x < PW; ++x) m_new = fmaxf(m_new, wmax[x][slot]);
                 const float corr = __expf(m[u] - m_new);
                 m[u] = m_new;
                 float psum = 0.f;
@@ -374,32 +374,32 @@ latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __
                     for (int i = 0; i < 4; ++i) acc[u][j][i] *= corr;
             }
             lam_lds_barrier();
-            // ---- weights times latents, two 32-key steps at a time; the next two are asked for as soon as these have
+            // ---- weights times latents, VH 32-key steps at a time; the next are asked for as soon as these have
             //      been read
 #pragma unroll
-            for (int pair = 0; pair < LAM_PW / 4; ++pair) {
+            for (int pair = 0; pair < PW / 2 / VH; ++pair) {
 #pragma unroll
-                for (int half = 0; half < 2; ++half)
+                for (int half = 0; half < VH; ++half)
 #pragma unroll
-                    for (int u = 0; u < LAM_TT; ++u) {
+                    for (int u = 0; u < TT; ++u) {
                         if (!live[u]) continue;
-                        const int at = (2 * pair + half) * 32 + quad * 8;
+                        const int at = (VH * pair + half) * 32 + quad * 8;
                         const lam_bf16x8 ph = *reinterpret_cast<const lam_bf16x8*>(&p_hi[u * 16 + col][at]);
                         const lam_bf16x8 pl = *reinterpret_cast<const lam_bf16x8*>(&p_lo[u * 16 + col][at]);
 #pragma unroll
                         for (int j = 0; j < CT; ++j)
-                            if (w + LAM_PW * j < tiles_c) {
+                            if (w + PW * j < tiles_c) {
                                 acc[u][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j][half], ph, acc[u][j], 0, 0, 0);
                                 acc[u][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j][half], pl, acc[u][j], 0, 0, 0);
                             }
                     }
-                if (pair + 1 < LAM_PW / 4) load_values(kb, pair + 1);
+                if (pair + 1 < PW / 2 / VH) load_values(kb, pair + 1);
             }
         }
         // ---- the slots' sums (the lane groups of a wavefront, then the wavefronts; wmax is free again) and the output
         __syncthreads();
 #pragma unroll
-        for (int u = 0; u < LAM_TT; ++u) {
+        for (int u = 0; u < TT; ++u) {
             float v = lsum[u];
             v += __shfl_xor(v, 16, 64);
             v += __shfl_xor(v, 32, 64);
@@ -407,16 +407,16 @@ latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __
         }
         __syncthreads();
 #pragma unroll
-        for (int u = 0; u < LAM_TT; ++u) {
+        for (int u = 0; u < TT; ++u) {
             if (!live[u] || head >= heads) continue;
             const int slot = u * 16 + col;
             float total = 0.f;
 #pragma unroll
-            for (int x = 0; x < LAM_PW; ++x) total += wmax[x][slot];
+            for (int x = 0; x < PW; ++x) total += wmax[x][slot];
             const float inv = 1.0f / total;
 #pragma unroll
             for (int j = 0; j < CT; ++j) {
-                const int ct = w + LAM_PW * j;
+                const int ct = w + PW * j;
                 if (ct >= tiles_c) continue;
                 lam_bf16x4 o;
 #pragma unroll
@@ -480,22 +480,25 @@ extern "C" int somi_latent_attention_mfma(const void* queries, const void* laten
     int page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
     if (portions) {
-        // prompt portions: LAM_TT tokens a workgroup, no key splits
+        // prompt portions: several tokens a workgroup, no key splits
         SOMI_REQUIRE(splits == 1, "latent_attention_mfma: prompt portions take no key splits");
-        const dim3 groups(ceil_div(n_tokens, LAM_TT), ceil_div(heads, 16));
-#define LAM_PORTION(STEPS, CT)                                                                                          \
+#define LAM_PORTION(STEPS, CT, TT, PW, WPS)                                                                            \
     do {                                                                                                                \
-        const size_t lds = (size_t)16 * LAM_TT * ((STEPS * 32 + 8) * 2 + (LAM_PKEYS + 8) * 4 + LAM_PW * 4);             \
-        hipError_t err = hipFuncSetAttribute((const void*)latent_attention_portion_kernel<STEPS, CT>,                   \
+        const dim3 groups(ceil_div(n_tokens, TT), ceil_div(heads, 16));                                                 \
+        const size_t lds = (size_t)16 * TT * ((STEPS * 32 + 8) * 2 + (16 * PW + 8) * 4 + PW * 4);                       \
+        hipError_t err = hipFuncSetAttribute((const void*)latent_attention_portion_kernel<STEPS, CT, TT, PW, WPS>,      \
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
         if (err != hipSuccess) return somi_fail("latent_attention_mfma: %s", hipGetErrorString(err));                   \
-        hipLaunchKernelGGL((latent_attention_portion_kernel<STEPS, CT>), groups, dim3(64 * LAM_PW), lds, stream,                \
-                           (const bf16*)queries, (const bf16*)latent, (const bf16*)latent_t, block_table, max_blocks,  \
-                           token_entry, positions, n_tokens, heads, rank, D, page_shift, scale, sink, (bf16*)out);       \
+        hipLaunchKernelGGL((latent_attention_portion_kernel<STEPS, CT, TT, PW, WPS>), groups, dim3(64 * PW), lds,       \
+                           stream, (const bf16*)queries, (const bf16*)latent, (const bf16*)latent_t, block_table,       \
+                           max_blocks, token_entry, positions, n_tokens, heads, rank, D, page_shift, scale, sink,      \
+                           (bf16*)out);                                                                                 \
     } while (0)
-        if (D <= 128 && rank <= 128) LAM_PORTION(4, 1);
-        else if (D <= 256 && rank <= 256) LAM_PORTION(8, 2);
-        else LAM_PORTION(18, 4);
+        // the widest rows: two tokens and four wavefronts a workgroup, two workgroups a compute unit (four tokens and
+        // eight wavefronts would not fit a wavefront's sums, fragments in flight and scores into its registers)
+        if (D <= 128 && rank <= 128) LAM_PORTION(4, 2, 2, 4, 2);
+        else if (D <= 256 && rank <= 256) LAM_PORTION(8, 4, 2, 4, 2);
+        else LAM_PORTION(18, 8, 2, 4, 2);
 #undef LAM_PORTION
         SOMI_LAUNCH_CHECK("latent_attention_portion");
         return 0;
