@@ -35,7 +35,8 @@ extern "C" int somi_gla_alpha(float* z, float tau, int64_t count, hipStream_t st
 }
 
 // ------------------------------------------------------------------------------------------------ the recurrence
-// A wavefront (a workgroup of its own) owns GLA_COLS columns of one (entry, head): lane = 4 * column + row group, and
+// A wavefront (a workgroup of its own) owns GLA_COLS columns of one (entry, head) (4 with 16 lanes a column, see the
+// kernel): lane = 4 * column + row group, and
 // row group g of the four holds the rows d = g * RPL .. g * RPL + RPL - 1 of its column in registers (rows past dim are
 // padding that stays zero).  The tokens' alpha, k, scaled q and v of the head go through LDS STAGE tokens at a time,
 // laid out so that a lane reads its rows four at a time.  The next tokens' values are asked of memory, as they are
@@ -69,24 +70,28 @@ template <typename T, int G> __device__ __forceinline__ GlaRaw<T, G> gla_load(co
 }
 
 // G: elements moved at a time, 4 where dim, vdim and the row strides are multiples of 4 and the rows aligned, else 1.
-template <typename T, int RPL, int G>
+// LPC: lanes that share a column of the state (4, or 16 where 4 would leave the device short of wavefronts: a wavefront
+// then owns 4 columns and a lane a sixteenth of the rows; the row groups' shares are added by two more data-parallel
+// moves, rotations inside the column's row of 16 lanes).
+template <typename T, int RPL, int G, int LPC>
 __global__ void __launch_bounds__(64)
 gla_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, int64_t row_stride,
                 const float* __restrict__ alpha, const int* __restrict__ entry_start,
                 const int* __restrict__ state_slots, float* __restrict__ state, int heads, int dim, int vdim,
                 float q_scale, float* __restrict__ o) {
-    constexpr int STAGE = RPL <= 16 ? 16 : (RPL <= 32 ? 8 : 4);       // tokens staged at a time
-    constexpr int ROWS = GLA_GROUPS * RPL;                             // padded rows of a head
+    constexpr int STAGE = RPL * LPC <= 64 ? 16 : (RPL * LPC <= 128 ? 8 : 4);   // tokens staged at a time
+    constexpr int COLS = 64 / LPC;                                     // columns of a wavefront
+    constexpr int ROWS = LPC * RPL;                                    // padded rows of a head
     constexpr int PIECES = STAGE * ROWS / G / 64;                      // pieces of G rows of each array a lane moves
-    constexpr int VPIECES = (STAGE * GLA_COLS / G + 63) / 64;          // pieces of G columns of v a lane moves
+    constexpr int VPIECES = (STAGE * COLS / G + 63) / 64;          // pieces of G columns of v a lane moves
     __shared__ __attribute__((aligned(16))) float sa[STAGE * ROWS];
     __shared__ __attribute__((aligned(16))) float sk[STAGE * ROWS];
     __shared__ __attribute__((aligned(16))) float sq[STAGE * ROWS];
-    __shared__ __attribute__((aligned(16))) float sv[STAGE * GLA_COLS];
-    __shared__ __attribute__((aligned(16))) float so[STAGE * GLA_COLS];
+    __shared__ __attribute__((aligned(16))) float sv[STAGE * COLS];
+    __shared__ __attribute__((aligned(16))) float so[STAGE * COLS];
     const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int col0 = blockIdx.z * GLA_COLS;
-    const int colidx = lane / GLA_GROUPS, group = lane % GLA_GROUPS;
+    const int col0 = blockIdx.z * COLS;
+    const int colidx = lane / LPC, group = lane % LPC;
     const int col = col0 + colidx;
     const bool live = col < vdim;
     const int t0 = entry_start[e], t1 = entry_start[e + 1];
@@ -115,8 +120,8 @@ gla_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __res
 #pragma unroll
         for (int j = 0; j < VPIECES; ++j) {
             const int piece = lane + 64 * j;
-            const int t = min(base + piece / (GLA_COLS / G), t1 - 1);
-            const int c = min(col0 + G * (piece % (GLA_COLS / G)), vdim - G);
+            const int t = min(base + piece / (COLS / G), t1 - 1);
+            const int c = min(col0 + G * (piece % (COLS / G)), vdim - G);
             rv[j] = gla_load<T, G>(v + (int64_t)t * row_stride + (int64_t)h * vdim + c);
         }
     };
@@ -143,8 +148,8 @@ gla_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __res
 #pragma unroll
         for (int j = 0; j < VPIECES; ++j) {
             const int piece = lane + 64 * j;
-            if (piece < STAGE * GLA_COLS / G) {
-                const int tt = piece / (GLA_COLS / G), c = G * (piece % (GLA_COLS / G));
+            if (piece < STAGE * COLS / G) {
+                const int tt = piece / (COLS / G), c = G * (piece % (COLS / G));
 #pragma unroll
                 for (int x = 0; x < G; ++x)
                     sv[piece * G + x] = (base + tt < t1 && col0 + c + x < vdim) ? to_float(rv[j].v[x]) : 0.f;
@@ -159,7 +164,7 @@ gla_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __res
             const float* a = sa + tt * ROWS + group * RPL;
             const float* kk = sk + tt * ROWS + group * RPL;
             const float* qq = sq + tt * ROWS + group * RPL;
-            const float vt = sv[tt * GLA_COLS + colidx];
+            const float vt = sv[tt * COLS + colidx];
             float part[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < RPL; i += 4) {
@@ -175,20 +180,24 @@ gla_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __res
             float acc = (part[0] + part[1]) + (part[2] + part[3]);
             acc += quad_swap<0xB1>(acc);           // the neighbour in the quad, then the other pair: the four row groups
             acc += quad_swap<0x4E>(acc);
-            if (group == 0) so[tt * GLA_COLS + colidx] = acc;
+            if (LPC == 16) {
+                acc += quad_swap<0x124>(acc);      // the quad four lanes on in the column's row of 16, then the pair of quads
+                acc += quad_swap<0x128>(acc);
+            }
+            if (group == 0) so[tt * COLS + colidx] = acc;
         }
         __syncthreads();                           // the reads, before the next tokens are staged; so is whole
-        // the stage's o: token lane / 4, columns 4 * (lane % 4) .. + 3
-        if (lane < STAGE * 4) {
-            const int tt = lane / 4, c = 4 * (lane % 4);
+        // the stage's o in pieces of 4 columns: token lane / (COLS / 4), columns 4 * (lane % (COLS / 4)) .. + 3
+        if (lane < STAGE * (COLS / 4)) {
+            const int tt = lane / (COLS / 4), c = 4 * (lane % (COLS / 4));
             if (tt < count) {
                 float* row = o + ((int64_t)(base + tt) * heads + h) * vdim + col0 + c;
                 if (G == 4) {
-                    if (col0 + c < vdim) *reinterpret_cast<gla_f32x4*>(row) = *reinterpret_cast<const gla_f32x4*>(so + tt * GLA_COLS + c);
+                    if (col0 + c < vdim) *reinterpret_cast<gla_f32x4*>(row) = *reinterpret_cast<const gla_f32x4*>(so + tt * COLS + c);
                 } else {
 #pragma unroll
                     for (int x = 0; x < 4; ++x)
-                        if (col0 + c + x < vdim) row[x] = so[tt * GLA_COLS + c + x];
+                        if (col0 + c + x < vdim) row[x] = so[tt * COLS + c + x];
                 }
             }
         }
@@ -206,40 +215,50 @@ gla_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __res
 // o: [n_tokens, heads, vdim] float32.
 extern "C" int somi_gla_scan(const void* q, const void* k, const void* v, int dtype, int64_t row_stride,
                              const float* alpha, const int* entry_start, const int* state_slots, float* state,
-                             int n_entries, int heads, int dim, int vdim, float q_scale, float* o,
+                             int n_entries, int heads, int dim, int vdim, float q_scale, int lanes, float* o,
                              hipStream_t stream) {
     SOMI_REQUIRE(n_entries >= 0 && heads > 0 && dim > 0 && vdim > 0, "gla_scan: bad sizes");
     SOMI_REQUIRE(dim <= 64 * GLA_GROUPS, "gla_scan: a key size of %d is more than the supported %d", dim, 64 * GLA_GROUPS);
     SOMI_REQUIRE(row_stride >= (int64_t)heads * dim && row_stride >= (int64_t)heads * vdim, "gla_scan: rows too narrow");
     SOMI_REQUIRE(heads <= 65535 && ceil_div(vdim, GLA_COLS) <= 65535, "gla_scan: too many heads or columns");
     if (n_entries == 0) return 0;
-    const dim3 grid(n_entries, heads, ceil_div(vdim, GLA_COLS));
-    const int rpl = ceil_div(dim, GLA_GROUPS);
+    // lanes a column: from the model's sizes and the device only, never from the step, so that a request's sums have one
+    // order in every batch; 16 where 4 would leave fewer than two wavefronts a compute unit for one request (and the
+    // rows are enough for 16 lanes)
+    SOMI_REQUIRE(lanes == 0 || lanes == 4 || lanes == 16, "gla_scan: %d lanes a column; 4 or 16", lanes);
+    const int lpc = lanes ? lanes : (heads * ceil_div(vdim, GLA_COLS) < 2 * somi_units() && dim >= 64 ? 16 : 4);
+    const dim3 grid(n_entries, heads, ceil_div(vdim, 64 / lpc));
+    const int rpl = lpc == 16 ? ceil_div(dim, 16) : ceil_div(dim, GLA_GROUPS);
     // four elements at a time where every piece of four is whole and aligned
     const bool wide = dim % 4 == 0 && vdim % 4 == 0 && row_stride % 4 == 0 && (uintptr_t)q % 16 == 0 && (uintptr_t)k % 8 == 0 &&
                       (uintptr_t)v % 8 == 0 && (uintptr_t)alpha % 16 == 0 && (uintptr_t)o % 16 == 0 &&
                       (dtype == SOMI_BF16 || ((uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0));
-#define GLA_LAUNCH(T, R)                                                                                              \
+#define GLA_LAUNCH(T, R, L)                                                                                           \
     do {                                                                                                              \
         if (wide)                                                                                                     \
-            hipLaunchKernelGGL((gla_scan_kernel<T, R, 4>), grid, dim3(64), 0, stream, (const T*)q, (const T*)k,       \
+            hipLaunchKernelGGL((gla_scan_kernel<T, R, 4, L>), grid, dim3(64), 0, stream, (const T*)q, (const T*)k,    \
                                (const T*)v, row_stride, alpha, entry_start, state_slots, state, heads, dim, vdim,     \
                                q_scale, o);                                                                           \
         else                                                                                                          \
-            hipLaunchKernelGGL((gla_scan_kernel<T, R, 1>), grid, dim3(64), 0, stream, (const T*)q, (const T*)k,       \
+            hipLaunchKernelGGL((gla_scan_kernel<T, R, 1, L>), grid, dim3(64), 0, stream, (const T*)q, (const T*)k,    \
                                (const T*)v, row_stride, alpha, entry_start, state_slots, state, heads, dim, vdim,     \
                                q_scale, o);                                                                           \
     } while (0)
 #define GLA_BY_ROWS(T)                                                                                                \
     do {                                                                                                              \
-        if (rpl <= 4) GLA_LAUNCH(T, 4);                                                                               \
-        else if (rpl <= 8) GLA_LAUNCH(T, 8);                                                                          \
-        else if (rpl <= 12) GLA_LAUNCH(T, 12);                                                                        \
-        else if (rpl <= 16) GLA_LAUNCH(T, 16);                                                                        \
-        else if (rpl <= 24) GLA_LAUNCH(T, 24);                                                                        \
-        else if (rpl <= 32) GLA_LAUNCH(T, 32);                                                                        \
-        else if (rpl <= 48) GLA_LAUNCH(T, 48);                                                                        \
-        else GLA_LAUNCH(T, 64);                                                                                       \
+        if (lpc == 16) {                                                                                              \
+            if (rpl <= 4) GLA_LAUNCH(T, 4, 16);                                                                       \
+            else if (rpl <= 8) GLA_LAUNCH(T, 8, 16);                                                                  \
+            else if (rpl <= 12) GLA_LAUNCH(T, 12, 16);                                                                \
+            else GLA_LAUNCH(T, 16, 16);                                                                               \
+        } else if (rpl <= 4) GLA_LAUNCH(T, 4, 4);                                                                     \
+        else if (rpl <= 8) GLA_LAUNCH(T, 8, 4);                                                                       \
+        else if (rpl <= 12) GLA_LAUNCH(T, 12, 4);                                                                     \
+        else if (rpl <= 16) GLA_LAUNCH(T, 16, 4);                                                                     \
+        else if (rpl <= 24) GLA_LAUNCH(T, 24, 4);                                                                     \
+        else if (rpl <= 32) GLA_LAUNCH(T, 32, 4);                                                                     \
+        else if (rpl <= 48) GLA_LAUNCH(T, 48, 4);                                                                     \
+        else GLA_LAUNCH(T, 64, 4);                                                                                    \
     } while (0)
     if (dtype == SOMI_F32) GLA_BY_ROWS(float);
     else if (dtype == SOMI_BF16) GLA_BY_ROWS(bf16);

@@ -8,7 +8,7 @@
 // dtype.
 #include "common.h"
 
-#define CONV_MAX_TAPS 9
+#define CONV_MAX_TAPS 17
 
 template <typename TO>
 __global__ void __launch_bounds__(256)

@@ -827,10 +827,11 @@ def gla_alpha_(z: torch.Tensor, tau: float) -> torch.Tensor:
 
 
 def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, alpha: torch.Tensor, entry_start: torch.Tensor,
-             state_slots: torch.Tensor, state: torch.Tensor, q_scale: float) -> torch.Tensor:
+             state_slots: torch.Tensor, state: torch.Tensor, q_scale: float, lanes: int = 0) -> torch.Tensor:
     """The recurrence S <- diag(alpha_t) S + k_t v_t^T, o_t = S^T (q_t * q_scale) per head over the tokens of every entry,
     from and into ``state[state_slots[e]]`` ([slots, heads, dim, vdim] float32) -> o [N, heads, vdim] float32.
-    q, k: [N, heads * dim] and v: [N, heads * vdim], views of one matrix (one row stride)."""
+    q, k: [N, heads * dim] and v: [N, heads * vdim], views of one matrix (one row stride).  ``lanes``: lanes that share a
+    column of the state (4 or 16; 0: the launcher chooses by the model's sizes and the device)."""
     slots, heads, dim, vdim = state.shape
     _need(state, "recurrent state", torch.float32)
     n = q.shape[0]
@@ -845,7 +846,7 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, alpha: torch.Ten
     o = torch.empty((n, heads, vdim), dtype=torch.float32, device=q.device)
     _check(library().somi_gla_scan(_ptr(q), _ptr(k), _ptr(v), dtype_code(q.dtype), ctypes.c_int64(q.stride(0)),
                                    _ptr(alpha), _ptr(entry_start), _ptr(state_slots), _ptr(state), entries, heads, dim,
-                                   vdim, ctypes.c_float(q_scale), _ptr(o), _stream()))
+                                   vdim, ctypes.c_float(q_scale), int(lanes), _ptr(o), _stream()))
     return o
 
 
@@ -1273,7 +1274,7 @@ def layernorm_add(h: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, bias: 
     return copy
 
 
-CONV_MAX_TAPS = 9
+CONV_MAX_TAPS = 17
 
 
 def input_conv(h: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, step, out_dtype: torch.dtype) -> torch.Tensor:

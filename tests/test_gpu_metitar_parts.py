@@ -126,7 +126,7 @@ def test_layer_norm_and_its_add_into_the_stream(dtype, width):
 
 # ------------------------------------------------------------------------------------------ the input convolution
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("taps,width", [(1, 24), (2, 100), (4, 96), (5, 300), (9, 8)])
+@pytest.mark.parametrize("taps,width", [(1, 24), (2, 100), (4, 96), (5, 300), (9, 8), (17, 40)])
 def test_input_convolution_whole_cut_and_side_by_side(dtype, taps, width):
     gen = torch.Generator().manual_seed(taps)
     conv = build_part("input_conv", PartSpec("short_causal", {"hidden_size": width, "taps": taps}), prefix="c")
@@ -392,3 +392,33 @@ def test_per_head_products(dtype, pads, heads, n_out, k, rows):
     want = torch.einsum("thk,hok->tho", x[:, :, :k], w)
     check(out[:, :, :n_out].float().cpu(), want, dtype, 8)
     assert float(out[:, :, n_out:].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("lanes", [4, 16])
+@pytest.mark.parametrize("heads,dim,vdim", [(2, 64, 32), (1, 128, 64), (3, 100, 20), (2, 16, 8), (1, 256, 12)])
+def test_the_recurrence_with_either_number_of_lanes_a_column(lanes, heads, dim, vdim):
+    """The recurrence kernel spreads a column of the state over 4 or over 16 lanes; both against the recurrence written
+    out, from a state that is not empty, with two requests of unequal length in one launch."""
+    gen = torch.Generator().manual_seed(dim + lanes)
+    n = 37
+    rows = torch.randn(n, 2 * heads * dim + heads * vdim, generator=gen)
+    keep = torch.rand(n, heads * dim, generator=gen)
+    state = torch.randn(3, heads, dim, vdim, generator=gen)
+    starts = torch.tensor([0, 30, n], dtype=torch.int32)
+    slots = torch.tensor([2, 0], dtype=torch.int32)
+    qk = heads * dim
+    device_rows, device_state = rows.to(DEV), state.clone().to(DEV)
+    got = ops.gla_scan(device_rows[:, :qk], device_rows[:, qk:2 * qk], device_rows[:, 2 * qk:], keep.to(DEV), starts.to(DEV),
+                       slots.to(DEV), device_state, 0.5, lanes=lanes).cpu()
+    want = torch.zeros(n, heads, vdim)
+    after = state.clone()
+    for entry, slot in enumerate(slots.tolist()):
+        s = after[slot]
+        for t in range(int(starts[entry]), int(starts[entry + 1])):
+            q, k = rows[t, :qk].view(heads, dim), rows[t, qk:2 * qk].view(heads, dim)
+            v = rows[t, 2 * qk:].view(heads, vdim)
+            s = keep[t].view(heads, dim, 1) * s + k[:, :, None] * v[:, None, :]
+            want[t] = torch.einsum("hkv,hk->hv", s, q * 0.5)
+        after[slot] = s
+    torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(device_state.cpu(), after, rtol=1e-4, atol=1e-4)
