@@ -178,7 +178,7 @@ def plain_latent(x, weights, config, kept=None):
     (8, 128, 64, 128, 512, 96, 16, None, None),
     (20, 16, 16, 16, 48, 32, 8, None, None),              # more heads than a workgroup's 16 query slots
     (37, 8, 8, 8, 24, 16, 16, 4, None),
-    (2, 16, 16, 16, 640, 32, 16, None, None),              # a latent wider than the matrix-core kernel takes
+    (2, 16, 16, 16, 656, 32, 16, None, None),              # a latent wider than the matrix-core kernel takes
 ])
 def test_latent_attention_against_the_plain_function(dtype, heads, dim, rot, vdim, rank, q_rank, page, dims, scaling):
     mixer, weights, config = latent_mixer(dtype, heads, dim, rot, vdim, rank, q_rank, (dim + rot) ** -0.5, page, dims=dims,
