@@ -174,3 +174,66 @@ extern "C" int somi_poly_norm(const float* z, const float* coef, float eps, void
     SOMI_LAUNCH_CHECK("poly_norm");
     return 0;
 }
+
+// xIELU: a unit with a quadratic positive side and an exponential negative side, two stored numbers (p, q) on the device:
+//
+//     z > 0:   softplus(p) z^2 + z / 2            z <= 0:   (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2.
+//
+// z: float32 sums of the product in front (its bias added); float32 arithmetic, rounded once.
+__device__ __forceinline__ float somi_softplus(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+
+template <typename TO>
+__global__ void __launch_bounds__(256)
+xielu_kernel(const float* __restrict__ z, const float* __restrict__ pq, TO* __restrict__ out, int64_t count) {
+    const float ap = somi_softplus(pq[0]), an = 0.5f + somi_softplus(pq[1]);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t)gridDim.x * 256) {
+        const float v = z[i];
+        const float r = v > 0.f ? fmaf(ap * v, v, 0.5f * v) : fmaf(an, expm1f(v) - v, 0.5f * v);
+        out[i] = from_float<TO>(r);
+    }
+}
+
+extern "C" int somi_xielu(const float* z, const float* pq, void* out, int out_dtype, int64_t count, hipStream_t stream) {
+    SOMI_REQUIRE(count >= 0, "xielu: bad sizes");
+    if (count == 0) return 0;
+    const int grid = (int)(ceil_div64(count, 256) < 65536 ? ceil_div64(count, 256) : 65536);
+    if (out_dtype == SOMI_F32)
+        hipLaunchKernelGGL(xielu_kernel<float>, dim3(grid), dim3(256), 0, stream, z, pq, (float*)out, count);
+    else if (out_dtype == SOMI_BF16)
+        hipLaunchKernelGGL(xielu_kernel<bf16>, dim3(grid), dim3(256), 0, stream, z, pq, (bf16*)out, count);
+    else
+        return somi_fail("xielu: unknown dtype %d", out_dtype);
+    SOMI_LAUNCH_CHECK("xielu");
+    return 0;
+}
+
+// A sigmoid gate on rows: out = x * sigmoid(g) element by element; g: float32 sums of the gate's product, rows
+// g_stride apart; x and out: [n, width] of one type.
+template <typename T>
+__global__ void __launch_bounds__(256)
+sigmoid_gate_kernel(const T* __restrict__ x, const float* __restrict__ g, int64_t g_stride, T* __restrict__ out, int width,
+                    int64_t count) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t)gridDim.x * 256) {
+        const int64_t row = i / width;
+        const float gate = g[row * g_stride + (i - row * width)];
+        out[i] = from_float<T>(to_float(x[i]) / (1.0f + expf(-gate)));
+    }
+}
+
+extern "C" int somi_sigmoid_gate(const void* x, int dtype, const float* g, int64_t g_stride, void* out, int64_t n_rows,
+                                 int width, hipStream_t stream) {
+    SOMI_REQUIRE(n_rows >= 0 && width > 0 && g_stride >= width, "sigmoid_gate: bad sizes");
+    const int64_t count = n_rows * width;
+    if (count == 0) return 0;
+    const int grid = (int)(ceil_div64(count, 256) < 65536 ? ceil_div64(count, 256) : 65536);
+    if (dtype == SOMI_F32)
+        hipLaunchKernelGGL(sigmoid_gate_kernel<float>, dim3(grid), dim3(256), 0, stream, (const float*)x, g, g_stride,
+                           (float*)out, width, count);
+    else if (dtype == SOMI_BF16)
+        hipLaunchKernelGGL(sigmoid_gate_kernel<bf16>, dim3(grid), dim3(256), 0, stream, (const bf16*)x, g, g_stride,
+                           (bf16*)out, width, count);
+    else
+        return somi_fail("sigmoid_gate: unknown dtype %d", dtype);
+    SOMI_LAUNCH_CHECK("sigmoid_gate");
+    return 0;
+}

@@ -1330,17 +1330,28 @@ def head_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None 
     return out
 
 
-def latent_prepare(rows: torch.Tensor, q_rank: int, rank: int, rot: int, q_weight: torch.Tensor,
+PAIRINGS = {"half": 0, "neighbours": 1}      # which channels of a rotation turn together: i with i + dims / 2, or 2i with 2i + 1
+
+
+def pairing_code(pairing: str) -> int:
+    if pairing not in PAIRINGS:
+        raise KernelError(f"unknown pairing {pairing!r}; known: {sorted(PAIRINGS)}")
+    return PAIRINGS[pairing]
+
+
+def latent_prepare(rows: torch.Tensor, q_rank: int, rank: int, rot: int, q_weight: torch.Tensor | None,
                    c_weight: torch.Tensor | None, eps: float, inv_freq: torch.Tensor | None, rot_dims: int, amplitude: float,
                    positions: torch.Tensor, slots: torch.Tensor | None, latent: torch.Tensor | None,
-                   out_dtype: torch.dtype, latent_t: torch.Tensor | None = None) -> torch.Tensor:
+                   out_dtype: torch.dtype, latent_t: torch.Tensor | None = None, pairing: str = "half") -> torch.Tensor:
     """From float32 rows [query latent (q_rank) | latent as projected (rank) | shared key part (rot)]: the RMS-normed
-    query latent -> [N, q_rank] in ``out_dtype``; and, with ``latent`` ([pages, page, rank + rot]), the RMS-normed
+    query latent -> [N, q_rank] in ``out_dtype`` (without ``q_weight`` the first ``q_rank`` values are the queries
+    themselves and are only rounded); and, with ``latent`` ([pages, page, rank + rot]), the RMS-normed
     latent and the rotated key part into the tokens' slots (``latent_t`` [pages, rank, page]: the latent once more,
     transposed inside its page)."""
     _need(rows, "projected rows", torch.float32)
     n = rows.shape[0]
-    _need(q_weight, "query latent's norm weight", torch.float32, (q_rank,))
+    if q_weight is not None:
+        _need(q_weight, "query latent's norm weight", torch.float32, (q_rank,))
     _need(positions, "positions", torch.int32, (n,))
     if latent is not None:
         _need(latent, "kept latents", out_dtype)
@@ -1357,31 +1368,39 @@ def latent_prepare(rows: torch.Tensor, q_rank: int, rank: int, rot: int, q_weigh
     q_latent = torch.empty((n, q_rank), dtype=out_dtype, device=rows.device)
     _check(library().somi_latent_prepare(_ptr(rows), ctypes.c_int64(rows.stride(0)), n, int(q_rank), int(rank), int(rot),
                                          _ptr(q_weight), _ptr(c_weight), ctypes.c_float(eps), _ptr(inv_freq), int(rot_dims),
-                                         ctypes.c_float(amplitude), _ptr(positions), _ptr(slots), _ptr(q_latent),
+                                         ctypes.c_float(amplitude), pairing_code(pairing), _ptr(positions), _ptr(slots),
+                                         _ptr(q_latent),
                                          _ptr(latent), _ptr(latent_t), latent.shape[1] if latent is not None else 0,
                                          dtype_code(out_dtype), _stream()))
     return q_latent
 
 
 def latent_place(q: torch.Tensor, heads: int, dim: int, rot: int, rank: int, inv_freq: torch.Tensor | None, rot_dims: int,
-                 amplitude: float, positions: torch.Tensor, queries: torch.Tensor) -> None:
-    """The rotated part of every head of q ([N, heads * (dim + rot)], head by head [dim | rot]) turned by its position
-    and written to ``queries[t, h, rank:]`` ([N, heads, rank + rot])."""
-    _need(q, "projected queries", None, (queries.shape[0], heads * (dim + rot)))
-    _need(queries, "query rows", q.dtype, (q.shape[0], heads, rank + rot))
+                 amplitude: float, positions: torch.Tensor, queries: torch.Tensor, pairing: str = "half") -> None:
+    """The rotated part of every head of q ([N, heads * (dim + rot)], head by head [dim | rot]; of the queries' type or
+    float32, and possibly the first columns of wider rows) turned by its position and written to ``queries[t, h,
+    rank:]`` ([N, heads, rank + rot])."""
+    if not isinstance(q, torch.Tensor) or not q.is_cuda or q.dim() != 2 or q.stride(1) != 1 or q.shape[1] != heads * (dim + rot):
+        raise KernelError(f"latent_place: projected queries must be rows of {heads * (dim + rot)} values on the GPU")
+    if q.dtype not in (torch.float32, queries.dtype):
+        raise KernelError(f"latent_place: projected queries are float32 or {queries.dtype}, got {q.dtype}")
+    _need(queries, "query rows", None, (q.shape[0], heads, rank + rot))
     _need(positions, "positions", torch.int32, (q.shape[0],))
     if rot_dims:
         _need(inv_freq, "rotation frequencies", torch.float32, (rot_dims // 2,))
-    _check(library().somi_latent_place(_ptr(q), dtype_code(q.dtype), q.shape[0], int(heads), int(dim), int(rot), int(rank),
-                                       _ptr(inv_freq), int(rot_dims), ctypes.c_float(amplitude), _ptr(positions),
-                                       _ptr(queries), _stream()))
+    _check(library().somi_latent_place(_ptr(q), dtype_code(q.dtype), ctypes.c_int64(q.stride(0)), dtype_code(queries.dtype),
+                                       q.shape[0], int(heads), int(dim), int(rot), int(rank),
+                                       _ptr(inv_freq), int(rot_dims), ctypes.c_float(amplitude), pairing_code(pairing),
+                                       _ptr(positions), _ptr(queries), _stream()))
 
 
 def latent_attention_plain(queries: torch.Tensor, latent: torch.Tensor, block_table: torch.Tensor, token_entry: torch.Tensor,
-                           positions: torch.Tensor, rank: int, scale: float, sink: torch.Tensor) -> torch.Tensor:
+                           positions: torch.Tensor, rank: int, scale: float, sink: torch.Tensor | None,
+                           window: int = 0) -> torch.Tensor:
     """Causal softmax attention with a sink over kept latents: queries [N, heads, rank + rot] against the rows of
     ``latent`` ([pages, page, rank + rot]) of each token's request up to its own position; the values are the rows' first
-    ``rank`` channels -> [N, heads, rank]."""
+    ``rank`` channels -> [N, heads, rank].  ``sink`` None: a softmax over the keys alone.  ``window``: how many keys a
+    token sees, itself included (0: all)."""
     _need(queries, "query rows")
     n, heads, width = queries.shape
     _need(latent, "kept latents", queries.dtype)
@@ -1390,12 +1409,15 @@ def latent_attention_plain(queries: torch.Tensor, latent: torch.Tensor, block_ta
     _need(block_table, "block table", torch.int32)
     _need(token_entry, "token entries", torch.int32, (n,))
     _need(positions, "positions", torch.int32, (n,))
-    _need(sink, "sinks", torch.float32, (heads,))
+    if sink is not None:
+        _need(sink, "sinks", torch.float32, (heads,))
+    if window < 0:
+        raise KernelError(f"latent_attention: a window of {window} keys")
     out = torch.empty((n, heads, rank), dtype=queries.dtype, device=queries.device)
     _check(library().somi_latent_attention_plain(_ptr(queries), dtype_code(queries.dtype), _ptr(latent), _ptr(block_table),
                                                  block_table.shape[1], _ptr(token_entry), _ptr(positions), n, heads,
-                                                 int(rank), width - int(rank), latent.shape[1], ctypes.c_float(scale),
-                                                 _ptr(sink), _ptr(out), _stream()))
+                                                 int(rank), width - int(rank), latent.shape[1], int(window),
+                                                 ctypes.c_float(scale), _ptr(sink), _ptr(out), _stream()))
     return out
 
 
@@ -1437,4 +1459,134 @@ def latent_attention_mfma(queries: torch.Tensor, latent: torch.Tensor, latent_t:
                                                 block_table.shape[1], _ptr(token_entry), _ptr(positions), n, heads,
                                                 int(rank), width - int(rank), latent.shape[1], ctypes.c_float(scale),
                                                 _ptr(sink), splits, 1 if portions else 0, _ptr(out), _ptr(part), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------------------------------ several residual streams
+HC_MAX_STREAMS = 8
+
+
+def hc_step(lanes: torch.Tensor, *, y: torch.Tensor | None = None, mix: torch.Tensor | None = None,
+            out_weights: torch.Tensor | None = None, read: bool = False, in_weights: torch.Tensor | None = None,
+            norm_weight: torch.Tensor | None = None, eps: float = 0.0, out_dtype: torch.dtype = torch.float32,
+            copies: int = 1) -> torch.Tensor | None:
+    """What lies between two sublayers of a layer with several residual streams, in one launch.  ``lanes``: [S, N, W]
+    float32, updated in place.  With ``y`` ([N, W], float32 or bfloat16): ``x_t <- sum_s mix[s, t] x_s + out_weights[t]
+    y`` for all t at once.  With ``read``: returns ``sum_s in_weights[s] x_s`` of the new streams (weights of 1 without
+    ``in_weights``), RMS-normed with ``norm_weight`` and ``eps`` if given, in ``out_dtype``, ``copies`` times over
+    ([copies, N, W]; [N, W] for one copy)."""
+    _need(lanes, "residual streams", torch.float32)
+    if lanes.dim() != 3:
+        raise KernelError(f"hc_step: the streams are [S, N, W], got {tuple(lanes.shape)}")
+    streams, n, width = lanes.shape
+    if y is not None:
+        _need(y, "sublayer output", None, (n, width))
+        _need(mix, "stream mix", torch.float32, (streams, streams))
+        _need(out_weights, "stream output weights", torch.float32, (streams,))
+    if in_weights is not None:
+        _need(in_weights, "stream input weights", torch.float32, (streams,))
+    if norm_weight is not None:
+        _need(norm_weight, "norm weight", torch.float32, (width,))
+    out = None
+    if read:
+        out = torch.empty((copies, n, width) if copies != 1 else (n, width), dtype=out_dtype, device=lanes.device)
+    elif y is None:
+        raise KernelError("hc_step: neither a write nor a read")
+    _check(library().somi_hc_step(_ptr(lanes), streams, ctypes.c_int64(n), width, _ptr(mix), _ptr(out_weights), _ptr(y),
+                                  dtype_code(y.dtype) if y is not None else 0, _ptr(in_weights), 1 if read else 0,
+                                  _ptr(norm_weight), ctypes.c_float(eps), _ptr(out), dtype_code(out_dtype), int(copies),
+                                  _stream()))
+    return out
+
+
+# ------------------------------------------------------------------------------------------ attention with mixed heads
+def mixed_attention_store(rows: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor | None,
+                          inv_freq: torch.Tensor | None, rot_dims: int, pairing: str, value_freq: torch.Tensor | None,
+                          value_pairing: str, heads: int, kv_heads: int, dim: int, vdim: int,
+                          k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, out_dtype: torch.dtype) -> torch.Tensor:
+    """From float32 rows [q (heads * dim) | k (kv_heads * dim) | v (kv_heads * vdim)] as projected: q with its first
+    ``rot_dims`` channels a head rotated -> [N, heads * dim] in ``out_dtype``; k rotated likewise and v, rotated over all
+    its channels with ``value_freq`` ([vdim / 2]) if given, into the tokens' slots of ``k_cache`` [pages, kv_heads, page,
+    dim] and ``v_cache`` [pages, kv_heads, page, vdim].  Without the caches the rows hold q only."""
+    _need(rows, "projected rows", torch.float32)
+    n = rows.shape[0]
+    _need(positions, "positions", torch.int32, (n,))
+    page = 0
+    if k_cache is not None:
+        _need(k_cache, "key pages", out_dtype)
+        pages, page = k_cache.shape[0], k_cache.shape[2]
+        if tuple(k_cache.shape) != (pages, kv_heads, page, dim):
+            raise KernelError(f"mixed_attention_store: key pages {tuple(k_cache.shape)} != [pages, {kv_heads}, page, {dim}]")
+        _need(v_cache, "value pages", out_dtype, (pages, kv_heads, page, vdim))
+        _need(slots, "slot mapping", torch.int32, (n,))
+    if rows.shape[1] != heads * dim + (kv_heads * (dim + vdim) if k_cache is not None else 0):
+        raise KernelError(f"mixed_attention_store: rows of {rows.shape[1]} values do not hold the projections")
+    if rot_dims:
+        _need(inv_freq, "rotation frequencies", torch.float32, (rot_dims // 2,))
+    if value_freq is not None:
+        _need(value_freq, "value rotation frequencies", torch.float32, (vdim // 2,))
+    q = torch.empty((n, heads * dim), dtype=out_dtype, device=rows.device)
+    _check(library().somi_mixed_attention_store(_ptr(rows), ctypes.c_int64(rows.stride(0)), n, _ptr(positions), _ptr(slots),
+                                                _ptr(inv_freq), int(rot_dims), pairing_code(pairing), _ptr(value_freq),
+                                                pairing_code(value_pairing), int(heads), int(kv_heads), int(dim), int(vdim),
+                                                _ptr(q), _ptr(k_cache), _ptr(v_cache), int(page), dtype_code(out_dtype),
+                                                _stream()))
+    return q
+
+
+def mixed_attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                          token_entry: torch.Tensor, positions: torch.Tensor, heads: int, window: int, scale: float,
+                          softcap: float, denominator_extra: float, talk: torch.Tensor | None,
+                          value_freq: torch.Tensor | None, value_pairing: str = "half") -> torch.Tensor:
+    """Attention of every token over its request's pages up to its own position (``window`` keys back, itself included;
+    0: all): scores ``scale q . k``, capped smoothly at ``softcap`` if > 0; a softmax per head whose denominator also
+    holds ``denominator_extra`` (0 or 1); the heads' weights mixed by ``talk`` ([heads, heads], to x from) if given; a
+    head's mixed weights times the values of its own key/value head; with ``value_freq`` the result turned back by the
+    query's position.  q: [N, heads * dim]; out: [N, heads * vdim]."""
+    _need(q, "queries")
+    n = q.shape[0]
+    _need(k_cache, "key pages", q.dtype)
+    pages, kv_heads, page, dim = k_cache.shape
+    if q.shape[1] != heads * dim or heads % kv_heads:
+        raise KernelError(f"mixed_attention: queries {tuple(q.shape)} do not fit {heads} heads over key pages {tuple(k_cache.shape)}")
+    _need(v_cache, "value pages", q.dtype)
+    if v_cache.dim() != 4 or tuple(v_cache.shape[:3]) != (pages, kv_heads, page):
+        raise KernelError(f"mixed_attention: value pages {tuple(v_cache.shape)} do not fit key pages {tuple(k_cache.shape)}")
+    vdim = v_cache.shape[3]
+    _need(block_table, "block table", torch.int32)
+    _need(token_entry, "token entries", torch.int32, (n,))
+    _need(positions, "positions", torch.int32, (n,))
+    if talk is not None:
+        _need(talk, "head mix", torch.float32, (heads, heads))
+    if value_freq is not None:
+        _need(value_freq, "value rotation frequencies", torch.float32, (vdim // 2,))
+    out = torch.empty((n, heads * vdim), dtype=q.dtype, device=q.device)
+    _check(library().somi_mixed_attention_plain(_ptr(q), dtype_code(q.dtype), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
+                                                block_table.shape[1], _ptr(token_entry), _ptr(positions), n, int(heads),
+                                                kv_heads, dim, vdim, page, int(window), ctypes.c_float(scale),
+                                                ctypes.c_float(softcap), ctypes.c_float(denominator_extra), _ptr(talk),
+                                                _ptr(value_freq), pairing_code(value_pairing), _ptr(out), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------------------------------ activations and gates
+def xielu(z: torch.Tensor, pq: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """softplus(p) z^2 + z / 2 for z > 0 and (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2 otherwise; z: float32; pq: the
+    two stored numbers, float32 on the device."""
+    _need(z, "rows", torch.float32)
+    _need(pq, "activation numbers", torch.float32, (2,))
+    out = torch.empty(z.shape, dtype=out_dtype, device=z.device)
+    _check(library().somi_xielu(_ptr(z), _ptr(pq), _ptr(out), dtype_code(out_dtype), ctypes.c_int64(z.numel()), _stream()))
+    return out
+
+
+def sigmoid_gate(x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """x * sigmoid(gate) element by element; x: [N, W]; gate: float32 [N, W], possibly columns of wider rows."""
+    _need(x, "gated rows")
+    n, width = x.shape
+    if not gate.is_cuda or gate.dtype != torch.float32 or tuple(gate.shape) != (n, width) or gate.stride(1) != 1:
+        raise KernelError(f"sigmoid_gate: the gate is float32 rows of {width} values on the GPU, got {tuple(gate.shape)} {gate.dtype}")
+    out = torch.empty_like(x)
+    _check(library().somi_sigmoid_gate(_ptr(x), dtype_code(x.dtype), _ptr(gate), ctypes.c_int64(gate.stride(0)), _ptr(out),
+                                       ctypes.c_int64(n), width, _stream()))
     return out

@@ -4,8 +4,10 @@ from __future__ import annotations
 
 import torch
 
+from ..kernels import linear as linear_kernels
 from ..kernels import ops
 from ..kernels.stages import stage
+from ..weights.spec import VECTOR, Init, WeightSpec
 from .base import Block, BorrowedCache, CompositeSpec, LayerCache, Part, PartSpec
 from .registry import build_part
 from .residual import ResidualStream
@@ -158,6 +160,99 @@ class OutputNormBlock(Block):
                 x = self.ffn_norm.add_normed(h, fed, dtype if self.token_input is not None else None)
         if self.token_input is not None:
             self.token_input.add_to(h, x, step, 1.0)
+
+
+class HyperConnectionBlock(Block):
+    """A pre-norm layer around ``streams`` residual streams instead of one.  For sublayer q (the mixer, then the
+    feed-forward) with its three tensors ``in`` [S], ``mix`` [S, S] (from, to) and ``out`` [S]:
+
+        u = sum_s in[s] x_s;     y = sublayer(norm_q(u));     x_t <- sum_s mix[s, t] x_s + out[t] y    (all t at once).
+
+    The streams are all equal to the embedded rows when the first such layer meets them, and what the model's final
+    norm reads is their sum.  ``connections`` False: no such tensors; one stream with in = mix = out = 1, the plain
+    residual sum.  Streams, their sums and the norms are float32; a sublayer's last product is computed into float32
+    rows, and one kernel does a sublayer's write and the next sublayer's read and norm.  A layer without a feed-forward
+    has the first sublayer only.  ``names``: the sub-prefixes of the two norms, the mixer, the feed-forward and the two
+    sets of connection tensors."""
+
+    DEFAULT_NAMES = {"mixer_norm": "norm1", "mixer": "mix", "ffn_norm": "norm2", "feed_forward": "mlp",
+                     "mixer_streams": "hc1", "ffn_streams": "hc2"}
+
+    def __init__(self, prefix: str, mixer: PartSpec, feed_forward: PartSpec | None, mixer_norm: PartSpec,
+                 ffn_norm: PartSpec | None = None, streams: int = 1, connections: bool = True,
+                 names: dict[str, str] | None = None) -> None:
+        super().__init__(prefix)
+        sub = dict(self.DEFAULT_NAMES)
+        sub.update(names or {})
+        self.sub = sub
+        self.streams, self.connections = int(streams), bool(connections)
+        if not 1 <= self.streams <= ops.HC_MAX_STREAMS or (not self.connections and self.streams != 1):
+            raise ValueError(f"{prefix}: 1 to {ops.HC_MAX_STREAMS} streams (one without connection tensors), got {streams}")
+        self.mixer_norm = build_part("norm", mixer_norm, prefix=self.name(sub["mixer_norm"]))
+        self.mixer = build_part("mixer", mixer, prefix=self.name(sub["mixer"]))
+        self.ffn_norm = self.feed_forward = None
+        if feed_forward is not None:
+            if ffn_norm is None:
+                raise ValueError(f"{prefix}: a feed-forward needs its norm")
+            self.ffn_norm = build_part("norm", ffn_norm, prefix=self.name(sub["ffn_norm"]))
+            self.feed_forward = build_part("feed_forward", feed_forward, prefix=self.name(sub["feed_forward"]))
+        for norm in (self.mixer_norm, self.ffn_norm):
+            if norm is not None and not (getattr(norm, "fusable", False) and hasattr(norm, "eps")):
+                raise ValueError(f"{prefix}: the kernel that reads the streams norms them by their root mean square")
+        self.graph_safe = all(getattr(part, "graph_safe", False) for part in self.parts())
+
+    def parts(self) -> list[Part]:
+        return [part for part in (self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward) if part is not None]
+
+    def _connection_names(self) -> list[str]:
+        subs = [self.sub["mixer_streams"]] + ([self.sub["ffn_streams"]] if self.feed_forward is not None else [])
+        return [self.name(s) for s in subs] if self.connections else []
+
+    def weight_specs(self):
+        specs = super().weight_specs()
+        s = self.streams
+        for base in self._connection_names():
+            specs += [WeightSpec(f"{base}.in", (s,), VECTOR, Init(1.0 / s, 0.1)),
+                      WeightSpec(f"{base}.out", (s,), VECTOR, Init(1.0, 0.1)),
+                      WeightSpec(f"{base}.mix", (s, s), VECTOR, Init(1.0 / s, 0.1))]
+        return specs
+
+    def load(self, fetch, runtime) -> None:
+        super().load(fetch, runtime)
+        self.links = []
+        for base in self._connection_names():
+            self.links.append((fetch(f"{base}.in"), fetch(f"{base}.mix").contiguous(), fetch(f"{base}.out")))
+        if not self.connections:
+            one = torch.ones((1,), dtype=torch.float32, device=runtime.device)
+            self.links = [(one, one.view(1, 1), one)] * 2
+
+    def forward(self, stream: ResidualStream, step, cache: LayerCache | None) -> None:
+        lanes = stream.fan_out(self.streams)
+        dtype = self.runtime.dtype
+        first, second = self.links[0], (self.links[1] if self.feed_forward is not None else None)
+        with stage("residual add, norm"):
+            x = ops.hc_step(lanes, read=True, in_weights=first[0], norm_weight=self.mixer_norm.weight,
+                            eps=self.mixer_norm.eps, out_dtype=dtype)
+        y = _float32_product(self.mixer.forward(x, step, cache))
+        if second is None:
+            with stage("residual add, norm"):
+                ops.hc_step(lanes, y=y, mix=first[1], out_weights=first[2])
+            return
+        with stage("residual add, norm"):
+            x = ops.hc_step(lanes, y=y, mix=first[1], out_weights=first[2], read=True, in_weights=second[0],
+                            norm_weight=self.ffn_norm.weight, eps=self.ffn_norm.eps, out_dtype=dtype)
+        y = _float32_product(self.feed_forward.forward(x, step))
+        with stage("residual add, norm"):
+            ops.hc_step(lanes, y=y, mix=second[1], out_weights=second[2])
+
+
+def _float32_product(y):
+    """A sublayer's output for the float32 streams: a promised product is computed into float32 rows, so that its
+    sums are not rounded before they are added; rows that exist stay as they are."""
+    if hasattr(y, "projection"):
+        with stage(y.projection.label):
+            return linear_kernels.linear(y.x, y.projection.weight, y.projection.bias, torch.float32)
+    return y
 
 
 def _rows(y):

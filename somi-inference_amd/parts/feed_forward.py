@@ -144,3 +144,64 @@ class PolyNormFF(FeedForward):
             a = ops.poly_norm(z, self.coefficients, self.eps, self.runtime.dtype)
         with stage(self.down.label):
             return linear_kernels.linear(a, self.down.weight, None, torch.float32)
+
+
+class ActivatedFF(FeedForward):
+    """y = down(act(up(x) + b_up)) + b_down without a gate, act an element-wise unit with stored numbers of its own.
+
+    ``activation`` "xielu": with the two stored numbers (p, q) of the ``act`` tensor,
+
+        act(z) = softplus(p) z^2 + z / 2                          for z > 0,
+                 (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2     for z <= 0.
+
+    The up product leaves float32 sums (bias added), the unit is float32 and rounded once to the compute dtype; the
+    down product leaves float32 sums for the residual streams."""
+    graph_safe = True
+
+    ROLES = {"up": "up", "down": "down", "act": "act"}
+    ACTIVATIONS = {"xielu": 2}          # name -> how many numbers it stores
+
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "xielu", bias: bool = True,
+                 names: dict[str, str] | None = None, suffix: str = "weight", bias_suffix: str = "bias") -> None:
+        super().__init__(prefix)
+        unknown = set(names or {}) - set(self.ROLES)
+        if unknown:
+            raise ValueError(f"{prefix}: unknown tensor roles {sorted(unknown)}; known: {sorted(self.ROLES)}")
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"{prefix}: unknown activation {activation!r}; known: {sorted(self.ACTIVATIONS)}")
+        self.names = {**self.ROLES, **(names or {})}
+        self.suffix, self.bias_suffix = str(suffix), str(bias_suffix)
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.activation, self.bias = activation, bool(bias)
+
+    def _tensor(self, role: str) -> str:
+        return self.name(f"{self.names[role]}.{self.suffix}" if self.suffix else self.names[role])
+
+    def _bias(self, role: str) -> str:
+        return self.name(f"{self.names[role]}.{self.bias_suffix}")
+
+    def weight_specs(self) -> list[WeightSpec]:
+        h, i = self.hidden_size, self.intermediate_size
+        specs = [WeightSpec(self._tensor("up"), (i, h), MATRIX), WeightSpec(self._tensor("down"), (h, i), MATRIX),
+                 WeightSpec(self.name(self.names["act"]), (self.ACTIVATIONS[self.activation],), VECTOR, Init(0.3, 0.3))]
+        if self.bias:
+            specs += [WeightSpec(self._bias("up"), (i,), VECTOR), WeightSpec(self._bias("down"), (h,), VECTOR)]
+        return specs
+
+    def load(self, fetch: Fetch, runtime: Runtime) -> None:
+        super().load(fetch, runtime)
+        self.up = Projection(fetch(self._tensor("up")), fetch(self._bias("up")) if self.bias else None, label="up")
+        self.down = Projection(fetch(self._tensor("down")), fetch(self._bias("down")) if self.bias else None, label="down")
+        self.numbers = fetch(self.name(self.names["act"]))
+
+    def flops(self, tokens: int, attended: int) -> float:
+        return self.up.flops(tokens) + self.down.flops(tokens)
+
+    def forward(self, x, step=None):
+        if hasattr(x, "materialize"):
+            x = x.materialize()
+        with stage(self.up.label):
+            z = linear_kernels.linear(x, self.up.weight, self.up.bias, torch.float32)
+        with stage("activation"):
+            a = ops.xielu(z, self.numbers, self.runtime.dtype)
+        return self.down.deferred(a)

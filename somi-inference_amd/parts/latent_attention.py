@@ -17,6 +17,10 @@ softmax are float32 in both engines.
 
 A layer that ``shares_cache`` has no W_dkv: it reads the vectors an earlier layer kept (the plan's ``cache_from``) with
 its own U, V, queries and sink.
+
+Variants, each a parameter: no query latent (``q_rank`` None: ``q = W_q h``), no sink (a softmax over the keys alone), a
+``window`` of keys a token sees (itself included), a sigmoid gate on the concatenated heads before ``W_o`` (``sigmoid(W_g
+h)`` of the mixer's own input), and the rotation's pairing (what the position part says).
 """
 
 from __future__ import annotations
@@ -36,15 +40,21 @@ class LatentAttention(Mixer):
     graph_safe = True
     PORTION_TOKENS = 8     # a step whose longest entry has this many tokens runs the kernel that shares a workgroup among tokens
 
-    ROLES = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv",
-             "sink": "sink", "o": "o", "position": "rotary_emb"}
+    ROLES = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "q": "q", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk",
+             "uv": "uv", "sink": "sink", "g": "g", "o": "o", "position": "rotary_emb"}
 
     def __init__(self, prefix: str, hidden_size: int, num_heads: int, dim: int, rot_dim: int, value_dim: int, kv_rank: int,
-                 q_rank: int, scale: float, eps: float, position: PartSpec, shares_cache: bool = False,
-                 page_size: int | None = None, names: dict[str, str] | None = None, suffix: str = "weight") -> None:
+                 q_rank: int | None, scale: float, eps: float, position: PartSpec, shares_cache: bool = False,
+                 page_size: int | None = None, names: dict[str, str] | None = None, suffix: str = "weight",
+                 sink: bool = True, window: int | None = None, kept_window: "int | None | str" = "same",
+                 gate: bool = False) -> None:
         """``position``: the rotation of the ``rot_dim`` channels (a rotary encoding of head size ``rot_dim``, or none).
         ``names``: role -> the checkpoint's name under the prefix (``dq_norm``, ``dkv_norm`` and ``sink`` are whole
-        names; the matrices are followed by ``suffix`` unless it is empty)."""
+        names; the matrices are followed by ``suffix`` unless it is empty).  ``q_rank`` None: no query latent, the
+        queries are one product of the input (role ``q``).  ``sink`` False: no sink.  ``window``: the keys a token sees,
+        itself included (None: all).  ``kept_window``: how long a token's kept row stays in the cache, where layers that
+        read this layer's cache see further back than it does itself ("same": as long as ``window`` says; None: for
+        ever).  ``gate``: the concatenated heads are multiplied by ``sigmoid(W_g h)`` (role ``g``) before ``W_o``."""
         super().__init__(prefix)
         unknown = set(names or {}) - set(self.ROLES)
         if unknown:
@@ -53,13 +63,17 @@ class LatentAttention(Mixer):
         self.suffix = str(suffix)
         self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
         self.dim, self.rot_dim, self.value_dim = int(dim), int(rot_dim), int(value_dim)
-        self.kv_rank, self.q_rank = int(kv_rank), int(q_rank)
+        self.kv_rank, self.q_rank = int(kv_rank), (int(q_rank) if q_rank is not None else None)
         self.scale, self.eps = float(scale), float(eps)
         self.shares_cache = bool(shares_cache)
         self.page_size = int(page_size) if page_size else None
+        self.has_sink, self.has_gate = bool(sink), bool(gate)
+        self.window = int(window) if window else None
+        self.kept_window = self.window if kept_window == "same" else (int(kept_window) if kept_window else None)
+        if self.kept_window is not None and (self.window is None or self.window > self.kept_window):
+            raise ValueError(f"{prefix}: a token sees {self.window or 'all'} keys but rows are kept for {self.kept_window}")
         self.position = build_part("position", position, prefix=self.name(self.names["position"]))
-        if getattr(self.position, "pairing", "half") != "half":
-            raise ValueError(f"{prefix}: this part's kernels rotate channel j with j + rotary_dim / 2 only")
+        self.pairing = getattr(self.position, "pairing", "half")
         self.rot_dims = int(getattr(self.position, "rotary_dim", 0))
         if self.rot_dims > self.rot_dim:
             raise ValueError(f"{prefix}: {self.rot_dims} rotated channels do not fit a key part of {self.rot_dim}")
@@ -70,35 +84,46 @@ class LatentAttention(Mixer):
 
     def weight_specs(self) -> list[WeightSpec]:
         h, heads, rank = self.hidden_size, self.num_heads, self.kv_rank
-        specs = [
-            WeightSpec(self._matrix("dq"), (self.q_rank, h), MATRIX),
-            WeightSpec(self.name(self.names["dq_norm"]), (self.q_rank,), VECTOR, Init(1.0, 0.1)),
-            WeightSpec(self._matrix("uq"), (heads * (self.dim + self.rot_dim), self.q_rank), MATRIX),
-        ]
+        if self.q_rank is None:
+            specs = [WeightSpec(self._matrix("q"), (heads * (self.dim + self.rot_dim), h), MATRIX)]
+        else:
+            specs = [
+                WeightSpec(self._matrix("dq"), (self.q_rank, h), MATRIX),
+                WeightSpec(self.name(self.names["dq_norm"]), (self.q_rank,), VECTOR, Init(1.0, 0.1)),
+                WeightSpec(self._matrix("uq"), (heads * (self.dim + self.rot_dim), self.q_rank), MATRIX),
+            ]
         if not self.shares_cache:
             specs += [WeightSpec(self._matrix("dkv"), (rank + self.rot_dim, h), MATRIX),
                       WeightSpec(self.name(self.names["dkv_norm"]), (rank,), VECTOR, Init(1.0, 0.1))]
         specs += [
             WeightSpec(self._matrix("uk"), (heads * self.dim, rank), MATRIX),
             WeightSpec(self._matrix("uv"), (heads * self.value_dim, rank), MATRIX),
-            WeightSpec(self.name(self.names["sink"]), (heads,), VECTOR, Init(0.0, 1.0)),
-            WeightSpec(self._matrix("o"), (h, heads * self.value_dim), MATRIX),
         ]
+        if self.has_sink:
+            specs.append(WeightSpec(self.name(self.names["sink"]), (heads,), VECTOR, Init(0.0, 1.0)))
+        if self.has_gate:
+            specs.append(WeightSpec(self._matrix("g"), (heads * self.value_dim, h), MATRIX))
+        specs.append(WeightSpec(self._matrix("o"), (h, heads * self.value_dim), MATRIX))
         return specs + self.position.weight_specs()
 
     def load(self, fetch: Fetch, runtime: Runtime) -> None:
         super().load(fetch, runtime)
         self.position.load(fetch, runtime)
-        down = [fetch(self._matrix("dq"))] + ([] if self.shares_cache else [fetch(self._matrix("dkv"))])
-        self.down = Projection.stacked(down, label="dq/dkv")
-        self.q_norm = fetch(self.name(self.names["dq_norm"]))
+        # one product of the input for everything that reads it: [query latent or queries | latent and shared key part |
+        # gate], float32 sums, so that nothing is rounded before the norms, the rotation and the sigmoid
+        down = [fetch(self._matrix("q" if self.q_rank is None else "dq"))]
+        down += [] if self.shares_cache else [fetch(self._matrix("dkv"))]
+        down += [fetch(self._matrix("g"))] if self.has_gate else []
+        self.down = Projection.stacked(down, label="q/dkv/g" if self.q_rank is None else "dq/dkv")
+        self.q_width = self.num_heads * (self.dim + self.rot_dim) if self.q_rank is None else self.q_rank
+        self.q_norm = None if self.q_rank is None else fetch(self.name(self.names["dq_norm"]))
         self.c_norm = None if self.shares_cache else fetch(self.name(self.names["dkv_norm"]))
-        self.up_q = Projection(fetch(self._matrix("uq")), label="uq")
+        self.up_q = None if self.q_rank is None else Projection(fetch(self._matrix("uq")), label="uq")
         heads, rank = self.num_heads, self.kv_rank
         # U_h^T per head, [heads, rank, dim]: the query's plain part goes to the latent's side
         self.key_maps = fetch(self._matrix("uk")).view(heads, self.dim, rank).transpose(1, 2).contiguous()
         self.value_maps = fetch(self._matrix("uv")).view(heads, self.value_dim, rank).contiguous()
-        self.sink = fetch(self.name(self.names["sink"]))
+        self.sink = fetch(self.name(self.names["sink"])) if self.has_sink else None
         self.out = Projection(fetch(self._matrix("o")), label="o")
         table = self.position.rotation_table() if self.rot_dims else None
         self.inv_freq = table[0] if table is not None else None
@@ -108,26 +133,28 @@ class LatentAttention(Mixer):
         heads, rank = self.num_heads, self.kv_rank
         per_head = 2.0 * tokens * heads * rank * (self.dim + self.value_dim)
         attention = 2.0 * attended * heads * (2 * rank + self.rot_dim)
-        return self.down.flops(tokens) + self.up_q.flops(tokens) + per_head + attention + self.out.flops(tokens)
+        up_q = self.up_q.flops(tokens) if self.up_q is not None else 0.0
+        return self.down.flops(tokens) + up_q + per_head + attention + self.out.flops(tokens)
 
     # -------------------------------------------------------------------- cache
     def cache_spec(self) -> PagedSpec:
         """A token's row [c | r], and c once more transposed inside its page (consecutive positions of one channel
         adjacent: the operand layout of the weights-times-latents product on the matrix cores)."""
         return PagedSpec((PageTensor("latent", (PAGE, self.kv_rank + self.rot_dim)),
-                          PageTensor("latent_t", (self.kv_rank, PAGE))), None, self.page_size)
+                          PageTensor("latent_t", (self.kv_rank, PAGE))), self.kept_window, self.page_size)
 
     # ------------------------------------------------------------------ forward
     def attend(self, queries: torch.Tensor, latent: torch.Tensor, step, view, latent_t: torch.Tensor | None = None) -> torch.Tensor:
         """The weighted sums of the kept latents for ``queries`` [N, heads, rank + rot] (the plain part already on the
         latent's side) -> [N, heads, rank].  bfloat16 sizes the matrix-core kernel is built for take it (it reads the
         transposed pages ``latent_t``); float32 and other sizes take the plain kernel."""
-        if latent_t is not None and ops.latent_attention_mfma_supported(queries, latent, self.kv_rank):
+        if (latent_t is not None and self.window is None and self.sink is not None
+                and ops.latent_attention_mfma_supported(queries, latent, self.kv_rank)):
             return ops.latent_attention_mfma(queries, latent, latent_t, view.block_table, step.token_entry, step.positions,
                                              self.kv_rank, self.scale, self.sink, step.max_context,
                                              portions=step.max_entry_len >= self.PORTION_TOKENS)
         return ops.latent_attention_plain(queries, latent, view.block_table, step.token_entry, step.positions,
-                                          self.kv_rank, self.scale, self.sink)
+                                          self.kv_rank, self.scale, self.sink, window=self.window or 0)
 
     def forward(self, x, step, cache: LayerCache | None):
         if cache is None or "latent" not in cache.tensors:
@@ -143,21 +170,26 @@ class LatentAttention(Mixer):
         with stage(self.down.label):
             rows = linear_kernels.linear(x, self.down.weight, None, torch.float32)
         with stage("latent norms, rotation, cache write"):
-            q_latent = ops.latent_prepare(rows, self.q_rank, rank, rot, self.q_norm, self.c_norm, self.eps, self.inv_freq,
+            q_latent = ops.latent_prepare(rows, self.q_width, rank, rot, self.q_norm, self.c_norm, self.eps, self.inv_freq,
                                           self.rot_dims, self.amplitude, step.positions,
                                           None if self.shares_cache else view.slot_mapping,
                                           None if self.shares_cache else latent, dtype,
-                                          None if self.shares_cache else latent_t)
-        q = self.up_q(q_latent)
+                                          None if self.shares_cache else latent_t, pairing=self.pairing)
+        # without a query latent the rows' first columns are the queries: their plain part as rounded by the kernel
+        # above, their rotated part straight from the float32 sums
+        q = self.up_q(q_latent) if self.up_q is not None else q_latent
         with stage("queries to the latent's side"):
             queries = torch.empty((n, heads, rank + rot), dtype=dtype, device=q.device)
             ops.head_linear(q.view(n, heads, self.dim + rot)[:, :, :self.dim], self.key_maps, out=queries[:, :, :rank])
             if rot:
-                ops.latent_place(q, heads, self.dim, rot, rank, self.inv_freq, self.rot_dims, self.amplitude,
-                                 step.positions, queries)
+                ops.latent_place(q if self.up_q is not None else rows[:, :self.q_width], heads, self.dim, rot, rank,
+                                 self.inv_freq, self.rot_dims, self.amplitude, step.positions, queries, pairing=self.pairing)
         with stage("attention"):
             mixed = self.attend(queries, latent, step, view, latent_t)
         with stage("values from the latent"):
             values = ops.head_linear(mixed, self.value_maps).view(n, heads * self.value_dim)
+        if self.has_gate:
+            with stage("output gate"):
+                values = ops.sigmoid_gate(values, rows[:, rows.shape[1] - heads * self.value_dim:])
         with stage(self.out.label):
             return linear_kernels.linear(values, self.out.weight, None, torch.float32)

@@ -26,14 +26,32 @@ class ResidualStream:
         assert h.dtype == torch.float32 and h.dim() == 2
         self.h = h
         self._pending: torch.Tensor | DeferredProduct | None = None
+        self.lanes: torch.Tensor | None = None      # [S, N, H] float32 once a layer keeps several streams side by side
+
+    def fan_out(self, count: int) -> torch.Tensor:
+        """The stream as ``count`` streams side by side, ``[count, N, H]`` float32, all equal to ``h`` when they are
+        made.  From then on the layers' arrangements update them in place, ``settle()`` gives their sum, and the
+        single-stream calls (``add``, ``normed``) are refused."""
+        if self.lanes is None:
+            h = self.settle()
+            self.lanes = ops.hc_step(h.unsqueeze(0), read=True, copies=count).view(count, *h.shape)
+        if self.lanes.shape[0] != count:
+            raise ValueError(f"the stream was fanned out into {self.lanes.shape[0]} streams, a layer asks for {count}")
+        return self.lanes
+
+    def _single(self) -> None:
+        if self.lanes is not None:
+            raise RuntimeError("the stream runs as several streams side by side; this layer's arrangement knows one")
 
     def add(self, delta: "torch.Tensor | DeferredProduct") -> None:
         """Queue ``h += delta``."""
+        self._single()
         self.settle()
         self._pending = delta
 
     def normed(self, norm: Norm, lazy: bool = False) -> "torch.Tensor | NormedRows":
         """norm(h) after any queued add.  ``lazy``: the caller's consumer takes :class:`NormedRows`."""
+        self._single()
         if isinstance(self._pending, DeferredProduct):
             pending, self._pending = self._pending, None
             if lazy and getattr(norm, "fusable", False):
@@ -46,7 +64,10 @@ class ResidualStream:
             return norm.forward(self.h)
 
     def settle(self) -> torch.Tensor:
-        """Apply a queued add and return the float32 rows."""
+        """Apply a queued add and return the float32 rows (of several streams: their sum, the streams stay)."""
+        if self.lanes is not None:
+            with stage("residual add, norm"):
+                return ops.hc_step(self.lanes, read=True)
         if isinstance(self._pending, DeferredProduct):
             self._pending.add_to(self.h)
         elif self._pending is not None:
