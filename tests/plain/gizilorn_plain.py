@@ -179,3 +179,16 @@ def forward(config: dict, weights: dict, tokens: list[int], dtype=torch.float64)
         after.append(streams.sum(dim=0))
     x = rms(streams.sum(dim=0), eps) * w["final.norm"]
     return x @ w["head"].T, torch.stack(after)
+
+
+def load_folder(folder: str, dtype=torch.float32) -> tuple[dict, dict]:
+    """(weights, config) of a model folder, floating tensors in ``dtype``."""
+    import json
+    import os
+
+    from safetensors.torch import load_file
+    with open(os.path.join(folder, "config.json"), "r", encoding="utf-8") as handle:
+        config = json.load(handle)
+    weights = {k: (v.to(dtype) if v.is_floating_point() else v)
+               for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    return weights, config
