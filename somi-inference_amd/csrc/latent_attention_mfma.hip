@@ -37,8 +37,8 @@ __global__ void __launch_bounds__(256)
 latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __restrict__ latent,
                              const bf16* __restrict__ latent_t, const int* __restrict__ block_table, int max_blocks,
                              const int* __restrict__ token_entry, const int* __restrict__ positions, int n_tokens,
-                             int heads, int rank, int D, int page_shift, float scale, const float* __restrict__ sink,
-                             int splits, bf16* __restrict__ out, float* __restrict__ part) {
+                             int heads, int rank, int D, int page_shift, int window, float scale,
+                             const float* __restrict__ sink, int splits, bf16* __restrict__ out, float* __restrict__ part) {
     const int page_mask = (1 << page_shift) - 1;
     __shared__ float wmax[4][16];
     __shared__ float wsum[4][16];
@@ -54,11 +54,13 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
     const int p = positions[t];
     const int* table = block_table + (int64_t)token_entry[t] * max_blocks;
     const int steps = (D + 31) >> 5, tiles_c = rank >> 4;
-    // this split's keys: whole 64-key tiles of the token's p + 1 keys
-    const int tiles_all = (p + LAM_KEYS) / LAM_KEYS;
+    // this split's keys: whole 64-key tiles (aligned to absolute positions) of the keys lo .. p that the token sees
+    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const int first_tile = lo / LAM_KEYS;
+    const int tiles_all = (p + LAM_KEYS) / LAM_KEYS - first_tile;
     const int per = (tiles_all + splits - 1) / splits;
-    const int k_begin = split * per * LAM_KEYS;
-    const int k_end = min(p + 1, (split + 1) * per * LAM_KEYS);
+    const int k_begin = (first_tile + split * per) * LAM_KEYS;
+    const int k_end = min(p + 1, (first_tile + (split + 1) * per) * LAM_KEYS);
 
     // the slots' queries go to LDS once (rows padded by 16 bytes, so that the 16 rows of a fragment fall on different
     // banks): held in registers they would leave no room for loads that run ahead
@@ -75,8 +77,9 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
     lam_f32x4 acc[CT];
 #pragma unroll
     for (int j = 0; j < CT; ++j) acc[j] = lam_f32x4{0.f, 0.f, 0.f, 0.f};
-    float m = split == 0 ? (live ? sink[head] : 0.f) : -INFINITY;
-    float lsum = (split == 0 && w == 0 && quad == 0) ? 1.f : 0.f;
+    // without a sink the first tile, which holds a key that is seen, sets the maximum
+    float m = split == 0 ? (live ? (sink != nullptr ? sink[head] : -INFINITY) : 0.f) : -INFINITY;
+    float lsum = (split == 0 && sink != nullptr && w == 0 && quad == 0) ? 1.f : 0.f;
 
     // A tile's K fragments (this wavefront's 16 keys) and the transposed latents of the channel tiles it owns, as they
     // are stored: nothing touches them until the products that read them.
@@ -121,7 +124,7 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int key = kb + 16 * w + quad * 4 + i;
-            s4[i] = key < k_end ? sc[i] * scale : -INFINITY;
+            s4[i] = key >= lo && key < k_end ? sc[i] * scale : -INFINITY;
             mx = fmaxf(mx, s4[i]);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -129,20 +132,21 @@ latent_attention_mfma_kernel(const bf16* __restrict__ queries, const bf16* __res
         if (quad == 0) wmax[w][col] = mx;
         lam_lds_barrier();
         const float m_new = fmaxf(fmaxf(m, fmaxf(wmax[0][col], wmax[1][col])), fmaxf(wmax[2][col], wmax[3][col]));
-        const float corr = __expf(m - m_new);
+        const float m_ref = m_new == -INFINITY ? 0.f : m_new;   // nothing seen yet: every weight below is exp(-inf) = 0
+        const float corr = __expf(m - m_ref);
         m = m_new;
         float psum = 0.f;
-        lam_bf16x4 hi, lo;
+        lam_bf16x4 hi, low;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float pv = __expf(s4[i] - m_new);              // exp(-inf) = 0 for keys that are not seen
+            const float pv = __expf(s4[i] - m_ref);              // exp(-inf) = 0 for keys that are not seen
             psum += pv;
             hi[i] = (__bf16)pv;
-            lo[i] = (__bf16)(pv - (float)hi[i]);
+            low[i] = (__bf16)(pv - (float)hi[i]);
         }
         lsum = lsum * corr + psum;
         *reinterpret_cast<lam_bf16x4*>(&p_hi[col][16 * w + quad * 4]) = hi;
-        *reinterpret_cast<lam_bf16x4*>(&p_lo[col][16 * w + quad * 4]) = lo;
+        *reinterpret_cast<lam_bf16x4*>(&p_lo[col][16 * w + quad * 4]) = low;
         if (__any(corr != 1.0f)) {                               // only where some slot's maximum moved
 #pragma unroll
             for (int j = 0; j < CT; ++j)
@@ -230,8 +234,8 @@ __global__ void __launch_bounds__(64 * PW, WPS)
 latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __restrict__ latent,
                                 const bf16* __restrict__ latent_t, const int* __restrict__ block_table, int max_blocks,
                                 const int* __restrict__ token_entry, const int* __restrict__ positions, int n_tokens,
-                                int heads, int rank, int D, int page_shift, float scale, const float* __restrict__ sink,
-                                bf16* __restrict__ out) {
+                                int heads, int rank, int D, int page_shift, int window, float scale,
+                                const float* __restrict__ sink, bf16* __restrict__ out) {
     const int page_mask = (1 << page_shift) - 1;
     constexpr int VH = CT >= 8 ? 1 : 2;          // 32-key steps whose transposed latents are in registers at a time
     constexpr int SLOTS = 16 * TT, QROW = STEPS * 32 + 8, PROW = (16 * PW) + 8, NT = 64 * PW;
@@ -255,13 +259,17 @@ latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __
         while (r1 < count && token_entry[t0 + r1] == entry) ++r1;
         const int* table = block_table + (int64_t)entry * max_blocks;
         const int p_last = positions[t0 + r1 - 1];
-        int pos[TT];
+        int pos[TT], first[TT];              // a token sees the keys first[u] .. pos[u]
         bool live[TT];
 #pragma unroll
         for (int u = 0; u < TT; ++u) {
             live[u] = u >= r0 && u < r1;
             pos[u] = live[u] ? positions[t0 + u] : -1;
+            first[u] = window > 0 ? max(0, pos[u] - window + 1) : 0;
         }
+        // the walk starts at the tile (aligned to absolute positions) of the first key the run's first token sees
+        const int p_first = positions[t0 + r0];
+        const int kb0 = ((window > 0 ? max(0, p_first - window + 1) : 0) / (16 * PW)) * (16 * PW);
         for (int i = threadIdx.x; i < SLOTS * STEPS * 4; i += NT) {
             const int slot = i / (STEPS * 4), ch = (i % (STEPS * 4)) * 8;
             const int u = slot >> 4, h = hg * 16 + (slot & 15);
@@ -279,8 +287,8 @@ latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __
         for (int u = 0; u < TT; ++u) {
 #pragma unroll
             for (int j = 0; j < CT; ++j) acc[u][j] = lam_f32x4{0.f, 0.f, 0.f, 0.f};
-            m[u] = live[u] && head < heads ? sink[head] : 0.f;
-            lsum[u] = (live[u] && w == 0 && quad == 0) ? 1.f : 0.f;
+            m[u] = live[u] && head < heads ? (sink != nullptr ? sink[head] : -INFINITY) : 0.f;
+            lsum[u] = (live[u] && sink != nullptr && w == 0 && quad == 0) ? 1.f : 0.f;
         }
         lam_bf16x8 kf[STEPS], vf[CT][VH];
 #pragma unroll
@@ -310,8 +318,8 @@ latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __
                 }
             }
         };
-        load_keys(0);
-        for (int kb = 0; kb <= p_last; kb += (16 * PW)) {
+        load_keys(kb0);
+        for (int kb = kb0; kb <= p_last; kb += (16 * PW)) {
             load_values(kb, 0);
             lam_f32x4 sc[TT];
 #pragma unroll
@@ -340,7 +348,7 @@ latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int key = kb + 16 * w + quad * 4 + i;
-                    s4[u][i] = key <= pos[u] ? sc[u][i] * scale : -INFINITY;
+                    s4[u][i] = key <= pos[u] && key >= first[u] ? sc[u][i] * scale : -INFINITY;
                     mx = fmaxf(mx, s4[u][i]);
                 }
                 mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -354,13 +362,14 @@ latent_attention_portion_kernel(const bf16* __restrict__ queries, const bf16* __
                 float m_new = m[u];
 #pragma unroll
                 for (int x = 0; x < PW; ++x) m_new = fmaxf(m_new, wmax[x][slot]);
-                const float corr = __expf(m[u] - m_new);
+                const float m_ref = m_new == -INFINITY ? 0.f : m_new;    // nothing seen yet: the weights below are 0
+                const float corr = __expf(m[u] - m_ref);
                 m[u] = m_new;
                 float psum = 0.f;
                 lam_bf16x4 hi, lo;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const float pv = __expf(s4[u][i] - m_new);          // exp(-inf) = 0 for keys that are not seen
+                    const float pv = __expf(s4[u][i] - m_ref);          // exp(-inf) = 0 for keys that are not seen
                     psum += pv;
                     hi[i] = (__bf16)pv;
                     lo[i] = (__bf16)(pv - (float)hi[i]);
@@ -462,14 +471,15 @@ extern "C" int somi_latent_attention_mfma_supported(int rank, int rot, int page_
 }
 
 // queries: [n_tokens, heads, rank + rot] bfloat16; latent: [pages, page, rank + rot]; latent_t: [pages, rank, page];
-// block_table: [entries, max_blocks]; sink: [heads] float32; out: [n_tokens, heads, rank] bfloat16; part: a workspace of
-// n_tokens * heads * splits * (rank + 2) floats where splits > 1.
+// block_table: [entries, max_blocks]; sink: [heads] float32 or null for a softmax over the keys alone; window: the keys
+// a token sees, itself included (0: all); out: [n_tokens, heads, rank] bfloat16; part: a workspace of n_tokens * heads *
+// splits * (rank + 2) floats where splits > 1.
 extern "C" int somi_latent_attention_mfma(const void* queries, const void* latent, const void* latent_t,
                                           const int* block_table, int max_blocks, const int* token_entry,
                                           const int* positions, int n_tokens, int heads, int rank, int rot, int page_size,
-                                          float scale, const float* sink, int splits, int portions, void* out, float* part,
-                                          hipStream_t stream) {
-    SOMI_REQUIRE(n_tokens >= 0 && heads > 0 && max_blocks > 0 && splits >= 1, "latent_attention_mfma: bad sizes");
+                                          int window, float scale, const float* sink, int splits, int portions, void* out,
+                                          float* part, hipStream_t stream) {
+    SOMI_REQUIRE(n_tokens >= 0 && heads > 0 && max_blocks > 0 && splits >= 1 && window >= 0, "latent_attention_mfma: bad sizes");
     SOMI_REQUIRE(somi_latent_attention_mfma_supported(rank, rot, page_size),
                  "latent_attention_mfma: a latent of %d + %d in pages of %d is not what the kernel is built for", rank, rot,
                  page_size);
@@ -491,8 +501,8 @@ extern "C" int somi_latent_attention_mfma(const void* queries, const void* laten
         if (err != hipSuccess) return somi_fail("latent_attention_mfma: %s", hipGetErrorString(err));                   \
         hipLaunchKernelGGL((latent_attention_portion_kernel<STEPS, CT, TT, PW, WPS>), groups, dim3(64 * PW), lds,       \
                            stream, (const bf16*)queries, (const bf16*)latent, (const bf16*)latent_t, block_table,       \
-                           max_blocks, token_entry, positions, n_tokens, heads, rank, D, page_shift, scale, sink,      \
-                           (bf16*)out);                                                                                 \
+                           max_blocks, token_entry, positions, n_tokens, heads, rank, D, page_shift, window, scale,    \
+                           sink, (bf16*)out);                                                                               \
     } while (0)
         // the widest rows: two tokens and four wavefronts a workgroup, two workgroups a compute unit (four tokens and
         // eight wavefronts would not fit a wavefront's sums, fragments in flight and scores into its registers)
@@ -507,7 +517,7 @@ extern "C" int somi_latent_attention_mfma(const void* queries, const void* laten
 #define LAM_LAUNCH(STEPS, CT)                                                                                          \
     hipLaunchKernelGGL((latent_attention_mfma_kernel<STEPS, CT>), grid, dim3(256), 0, stream, (const bf16*)queries,     \
                        (const bf16*)latent, (const bf16*)latent_t, block_table, max_blocks, token_entry, positions,    \
-                       n_tokens, heads, rank, D, page_shift, scale, sink, splits, (bf16*)out, part)
+                       n_tokens, heads, rank, D, page_shift, window, scale, sink, splits, (bf16*)out, part)
     if (D <= 128 && rank <= 128) LAM_LAUNCH(4, 2);
     else if (D <= 256 && rank <= 256) LAM_LAUNCH(8, 4);
     else LAM_LAUNCH(18, 8);

@@ -13,7 +13,9 @@
 // the values.  Scores, softmax, mix, the weighted sum and both rotations are float32.
 //
 //   store    one workgroup a token: q rotated into the rows the attention reads, k rotated and v (rotated or not) into
-//            the token's slot of the pages.  k: [pages, kv_heads, page, dim], v: [pages, kv_heads, page, vdim]
+//            the token's slot of the pages.  k: [pages, kv_heads, page, dim]; v is transposed inside a page, [pages,
+//            kv_heads, vdim, page]: consecutive positions of one channel are adjacent, the operand layout of the
+//            weights-times-values product on the matrix cores
 //   plain    one workgroup a token, all heads: a wavefront takes a head at a time and its 64 lanes the keys of a
 //            64-key tile (tiles aligned to absolute positions), so a head's maximum and sum are wave reductions
 #include "common.h"
@@ -85,7 +87,7 @@ mixed_store_kernel(const float* __restrict__ rows, int64_t row_stride, const int
                 v = first ? v * c - other * s : v * c + other * s;
             }
             const int64_t page = slot / page_size, off = slot % page_size;
-            v_cache[((page * kv + h) * page_size + off) * vdim + ch] = from_float<T>(v);
+            v_cache[((page * kv + h) * vdim + ch) * page_size + off] = from_float<T>(v);
         }
     }
 }
@@ -127,7 +129,8 @@ __device__ __forceinline__ float mxa_dot(const float* __restrict__ q, const T* _
 }
 
 // LDS (floats): q [heads * dim] | talk [heads * heads] | ml [2 * heads] | P [heads * TILE] | W [heads * TILE] |
-// O [heads * vdim]; then int64 rowbase [TILE]: page * kv * page_size + offset of each key of the tile.
+// O [heads * vdim]; then int64 rowbase [TILE]: page * kv * page_size + offset of each key of the tile (what a key's
+// row of kv head 0 starts at, in rows of k; the transposed values are addressed from its two parts).
 template <typename T>
 __global__ void __launch_bounds__(MXA_NT)
 mixed_attention_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -210,10 +213,13 @@ mixed_attention_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_ca
             const int i = tid + r * MXA_NT;
             if (i < heads * vdim) {
                 const int h = i / vdim, d = i % vdim;
-                const int64_t head_off = (int64_t)(h / group) * page_size;
+                const int c = h / group;
                 float a = acc[r];
-                for (int j = j0; j <= j1; ++j)
-                    a = fmaf(W[h * MXA_TILE + j], to_float(v_cache[(rowbase[j] + head_off) * vdim + d]), a);
+                for (int j = j0; j <= j1; ++j) {
+                    // rowbase = page * kv * page_size + offset with offset < page_size
+                    const int64_t page = rowbase[j] / ((int64_t)kv * page_size), off = rowbase[j] % page_size;
+                    a = fmaf(W[h * MXA_TILE + j], to_float(v_cache[((page * kv + c) * vdim + d) * page_size + off]), a);
+                }
                 acc[r] = a;
             }
         }
@@ -240,7 +246,7 @@ mixed_attention_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_ca
     }
 }
 
-// q: [n_tokens, heads * dim] rotated; k_cache: [pages, kv, page, dim]; v_cache: [pages, kv, page, vdim]; block_table:
+// q: [n_tokens, heads * dim] rotated; k_cache: [pages, kv, page, dim]; v_cache: [pages, kv, vdim, page]; block_table:
 // [entries, max_blocks]; talk: [heads, heads] float32 (to, from) or null for no mix; v_freq: [vdim / 2] float32 or null
 // for values that are not rotated; extra: what is added to the softmax's denominator (0 or 1); out: [n_tokens, heads *
 // vdim].

@@ -1,0 +1,289 @@
+// Attention with mixed heads on the matrix cores (bfloat16): see mixed_attention.hip for what is computed.
+//
+// A workgroup (four wavefronts) serves `tq` consecutive tokens of the step and ALL their heads, because the mix needs
+// every head's weights of a (token, key) pair in one place.  For each key/value head c there is one tile of 16 query
+// slots: slot = token * rp + r holds head c * group + r of that token (rp: the power of two >= group; slots with r >=
+// group, or of tokens of another request, are dead).  Tokens of one request stand side by side with rising positions;
+// where the workgroup's tokens belong to several requests it takes them run by run.
+//
+//   first walk   wavefront w takes the key/value heads w, w + 4, ...; 16 keys at a time, S^T = K Q^T by `16x16x32`
+//                products (K fragments straight from the pages, Q fragments from LDS); a lane holds 4 keys of one slot
+//                and keeps a running maximum and sum of its own, joined over the lanes at the end: (m, l) of every slot
+//   second walk  32 keys at a time: the same scores again, p = exp(s - m) / l in float32 into LDS; then all threads mix,
+//                w_h = sum_g T[h, g] p_g, float32, and leave the mixed weights in LDS as two bfloat16 halves (w = hi + lo,
+//                so no weight is rounded to eight bits); then O^T = V^T W^T, the V^T fragments straight from the pages
+//                (values are stored transposed inside a page), each wavefront owning some (key/value head, 16 channels)
+//                tiles of the output
+//   end          the sums go through LDS, are turned back by the query's position where values were turned by theirs,
+//                and are written out
+//
+// Keys below a token's window may lie in pages the request has given back: they are read (finite values of whoever
+// holds the page now) and weigh exactly 0.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 mxm_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float mxm_f32x4;
+
+#define MXM_PROW 33            // floats a slot's 32 weights take in LDS (one more: slots fall on different banks)
+#define MXM_WROW 40            // bfloat16 a slot's 32 mixed weights take (rows stay 16-byte aligned)
+
+__device__ __forceinline__ float mxm_cap(float s, float cap, float inv_cap) {
+    return cap > 0.f ? cap * tanhf(s * inv_cap) : s;
+}
+
+template <int STEPS, int ACC>
+__global__ void __launch_bounds__(256)
+mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+                            const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_entry,
+                            const int* __restrict__ positions, int n_tokens, int heads, int kv, int dim, int vdim,
+                            int page_size, int window, float scale, float cap, float extra,
+                            const float* __restrict__ talk, const float* __restrict__ v_freq, int v_pairing, int rp,
+                            int tq, bf16* __restrict__ out) {
+    constexpr int QROW = STEPS * 32 + 8;
+    extern __shared__ __attribute__((aligned(16))) char mxm_lds[];
+    bf16* q_s = reinterpret_cast<bf16*>(mxm_lds);                                  // [kv][16][QROW]
+    float* ml = reinterpret_cast<float*>(q_s + (size_t)kv * 16 * QROW);            // [kv][16][2]
+    float* P = ml + (size_t)kv * 32;                                               // [kv][16][PROW]
+    float* talk_s = P + (size_t)kv * 16 * MXM_PROW;                                // [heads][heads]
+    bf16* w_hi = reinterpret_cast<bf16*>(talk_s + ((heads * heads + 3) & ~3));     // [kv][16][WROW]
+    bf16* w_lo = w_hi + (size_t)kv * 16 * MXM_WROW;
+    float* o_s = reinterpret_cast<float*>(mxm_lds);                                // [kv][16][vdim], over all of the above
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, col = lane & 15, quad = lane >> 4;
+    const int group = heads / kv, dts = vdim >> 4;
+    const int t0 = (int)blockIdx.x * tq;
+    const int count = min(tq, n_tokens - t0);
+    const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
+    const int my_u = col / rp, my_r = col % rp;          // the token and head-in-group of the slot this lane serves
+
+    for (int r0 = 0; r0 < count;) {
+        const int entry = token_entry[t0 + r0];
+        int r1 = r0 + 1;
+        while (r1 < count && token_entry[t0 + r1] == entry) ++r1;
+        const int* table = block_table + (int64_t)entry * max_blocks;
+        const int p_first = positions[t0 + r0], k_hi = positions[t0 + r1 - 1];
+        const int k_lo = window > 0 ? max(0, p_first - window + 1) : 0;
+        const int kb0 = k_lo & ~31;
+        const bool live = my_u >= r0 && my_u < r1 && my_r < group;
+        const int my_pos = live ? positions[t0 + my_u] : -1;
+        const int my_first = window > 0 ? max(0, my_pos - window + 1) : 0;
+
+        // ---- the mix (the end of a run writes over it) and the queries of the run's tokens, slot by slot
+        for (int i = tid; i < heads * heads; i += 256)
+            talk_s[i] = talk != nullptr ? talk[i] : (i / heads == i % heads ? 1.f : 0.f);
+        for (int i = tid; i < kv * 16 * STEPS * 4; i += 256) {
+            const int ch = (i % (STEPS * 4)) * 8, slot = (i / (STEPS * 4)) % 16, c = i / (STEPS * 4 * 16);
+            const int u = slot / rp, r = slot % rp;
+            mxm_bf16x8 v;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.f;
+            if (u >= r0 && u < r1 && r < group && ch < dim)
+                v = *reinterpret_cast<const mxm_bf16x8*>(q + ((int64_t)(t0 + u) * heads + c * group + r) * dim + ch);
+            *reinterpret_cast<mxm_bf16x8*>(q_s + ((size_t)c * 16 + slot) * QROW + ch) = v;
+        }
+        __syncthreads();
+
+        // scores of 16 keys from kb on against the 16 slots of key/value head c: the lane's 4 keys of its slot
+        auto scores = [&](int c, int kb, float (&s4)[4]) {
+            const int key_row = min(kb + col, k_hi);
+            const int64_t page = table[key_row / page_size];
+            const bf16* krow = k_cache + ((page * kv + c) * page_size + key_row % page_size) * dim;
+            const bf16* q_lane = q_s + ((size_t)c * 16 + col) * QROW + quad * 8;
+            mxm_f32x4 sc = mxm_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) {
+                const int ch = s * 32 + quad * 8;
+                mxm_bf16x8 kf;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) kf[e] = (__bf16)0.f;
+                if (ch < dim) kf = *reinterpret_cast<const mxm_bf16x8*>(krow + ch);
+                sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, *reinterpret_cast<const mxm_bf16x8*>(q_lane + s * 32), sc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = kb + quad * 4 + i;
+                s4[i] = live && key >= my_first && key <= my_pos ? mxm_cap(sc[i] * scale, cap, inv_cap) : -INFINITY;
+            }
+        };
+
+        // ---- first walk: every slot's maximum and sum
+        for (int c = w; c < kv; c += 4) {
+            float m = -INFINITY, l = 0.f;
+            for (int kb = kb0; kb <= k_hi; kb += 16) {
+                float s4[4];
+                scores(c, kb, s4);
+                const float mx = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
+                const float m_new = fmaxf(m, mx);
+                if (m_new > -INFINITY) {
+                    l = l * __expf(m - m_new) + ((__expf(s4[0] - m_new) + __expf(s4[1] - m_new)) +
+                                                (__expf(s4[2] - m_new) + __expf(s4[3] - m_new)));
+                    m = m_new;
+                }
+            }
+            // the four lanes of a slot, then the sink's share
+            float top = fmaxf(m, __shfl_xor(m, 16, 64));
+            top = fmaxf(top, __shfl_xor(top, 32, 64));
+            if (extra > 0.f) top = fmaxf(top, 0.f);
+            float part = top > -INFINITY ? l * __expf(m - top) : 0.f;
+            part += __shfl_xor(part, 16, 64);
+            part += __shfl_xor(part, 32, 64);
+            if (extra > 0.f) part += extra * __expf(-top);
+            if (quad == 0) {
+                ml[(c * 16 + col) * 2] = top;
+                ml[(c * 16 + col) * 2 + 1] = part;
+            }
+        }
+        __syncthreads();
+
+        // ---- second walk: the weights, their mix, the sum over the values
+        mxm_f32x4 acc[ACC];
+#pragma unroll
+        for (int a = 0; a < ACC; ++a) acc[a] = mxm_f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int kb = kb0; kb <= k_hi; kb += 32) {
+            for (int c = w; c < kv; c += 4) {
+                const float m = ml[(c * 16 + col) * 2], inv_l = live ? 1.0f / ml[(c * 16 + col) * 2 + 1] : 0.f;
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    float s4[4];
+                    scores(c, kb + half * 16, s4);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        P[((size_t)c * 16 + col) * MXM_PROW + half * 16 + quad * 4 + i] = live ? __expf(s4[i] - m) * inv_l : 0.f;
+                }
+            }
+            __syncthreads();
+            for (int i = tid; i < kv * 16 * 32; i += 256) {
+                const int j = i & 31, slot = (i >> 5) & 15, c = i >> 9;
+                const int u = slot / rp, r = slot % rp;
+                float mixed = 0.f;
+                if (u >= r0 && u < r1 && r < group) {
+                    const float* t_row = talk_s + (c * group + r) * heads;
+                    for (int cg = 0; cg < kv; ++cg) {
+                        const float* p_row = P + ((size_t)cg * 16 + u * rp) * MXM_PROW + j;
+                        for (int rg = 0; rg < group; ++rg) mixed = fmaf(t_row[cg * group + rg], p_row[rg * MXM_PROW], mixed);
+                    }
+                }
+                const bf16 hi = (bf16)mixed;
+                w_hi[((size_t)c * 16 + slot) * MXM_WROW + j] = hi;
+                w_lo[((size_t)c * 16 + slot) * MXM_WROW + j] = (bf16)(mixed - (float)hi);
+            }
+            __syncthreads();
+            // the lane's 8 keys lie in one page (pages hold a multiple of 8 tokens, the walk is aligned to 32)
+            const int key8 = min(kb + quad * 8, k_hi & ~7);
+            const int64_t page = table[key8 / page_size];
+            const int off = key8 % page_size;
+#pragma unroll
+            for (int a = 0; a < ACC; ++a) {
+                const int pair = w + 4 * a;
+                if (pair < kv * dts) {
+                    const int c = pair / dts, dt = pair % dts;
+                    const mxm_bf16x8 vf = *reinterpret_cast<const mxm_bf16x8*>(
+                        v_cache + (((page * kv + c) * vdim + dt * 16 + col) * page_size + off));
+                    const size_t at = ((size_t)c * 16 + col) * MXM_WROW + quad * 8;
+                    acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, *reinterpret_cast<const mxm_bf16x8*>(w_hi + at), acc[a], 0, 0, 0);
+                    acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, *reinterpret_cast<const mxm_bf16x8*>(w_lo + at), acc[a], 0, 0, 0);
+                }
+            }
+        }
+        // ---- the heads' outputs through LDS, turned back by the query's position
+        __syncthreads();
+#pragma unroll
+        for (int a = 0; a < ACC; ++a) {
+            const int pair = w + 4 * a;
+            if (pair < kv * dts) {
+                const int c = pair / dts, dt = pair % dts;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o_s[((size_t)c * 16 + col) * vdim + dt * 16 + quad * 4 + i] = acc[a][i];
+            }
+        }
+        __syncthreads();
+        for (int i = tid; i < kv * 16 * vdim; i += 256) {
+            const int d = i % vdim, slot = (i / vdim) % 16, c = i / (vdim * 16);
+            const int u = slot / rp, r = slot % rp;
+            if (u < r0 || u >= r1 || r >= group) continue;
+            const float* row = o_s + ((size_t)c * 16 + slot) * vdim;
+            float v = row[d];
+            if (v_freq != nullptr) {
+                const int half = vdim >> 1;
+                const bool first = v_pairing == 0 ? d < half : (d & 1) == 0;
+                const int pair = v_pairing == 0 ? (first ? d : d - half) : d >> 1;
+                const float other = row[v_pairing == 0 ? (first ? d + half : d - half) : (d ^ 1)];
+                const float angle = (float)positions[t0 + u] * v_freq[pair];
+                const float cs = cosf(angle), sn = sinf(angle);            // by -angle: the sine changes its sign
+                v = first ? v * cs + other * sn : v * cs - other * sn;
+            }
+            out[((int64_t)(t0 + u) * heads + c * group + r) * vdim + d] = (bf16)v;
+        }
+        __syncthreads();
+        r0 = r1;
+    }
+}
+
+static size_t mxm_lds_bytes(int steps, int heads, int kv, int vdim) {
+    const size_t walk = (size_t)kv * 16 * (steps * 32 + 8) * 2 + (size_t)kv * 32 * 4 + (size_t)kv * 16 * MXM_PROW * 4 +
+                        (size_t)((heads * heads + 3) & ~3) * 4 + (size_t)kv * 16 * MXM_WROW * 2 * 2;
+    const size_t end = (size_t)kv * 16 * vdim * 4;
+    return walk > end ? walk : end;
+}
+
+static int mxm_steps(int dim) { return dim <= 32 ? 1 : dim <= 64 ? 2 : dim <= 128 ? 4 : 8; }
+static int mxm_acc(int kv, int vdim) {
+    const int need = ceil_div(kv * (vdim / 16), 4);
+    return need <= 2 ? 2 : need <= 4 ? 4 : need <= 8 ? 8 : 16;
+}
+
+extern "C" int somi_mixed_attention_mfma_supported(int heads, int kv, int dim, int vdim, int page_size) {
+    if (heads <= 0 || kv <= 0 || heads % kv || heads / kv > 16 || dim <= 0 || dim % 8 || dim > 256 || vdim <= 0 ||
+        vdim % 16 || page_size <= 0 || page_size % 8)
+        return 0;
+    if (ceil_div(kv * (vdim / 16), 4) > 16) return 0;
+    return mxm_lds_bytes(mxm_steps(dim), heads, kv, vdim) <= 160 * 1024 ? 1 : 0;
+}
+
+// As somi_mixed_attention_plain, bfloat16 only.  portions != 0: the step holds prompt portions, and as many consecutive
+// tokens share a workgroup as their heads fill 16 query slots a key/value head; otherwise a workgroup serves one token.
+extern "C" int somi_mixed_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int* block_table,
+                                         int max_blocks, const int* token_entry, const int* positions, int n_tokens,
+                                         int heads, int kv, int dim, int vdim, int page_size, int window, float scale,
+                                         float cap, float extra, const float* talk, const float* v_freq, int v_pairing,
+                                         int portions, void* out, hipStream_t stream) {
+    SOMI_REQUIRE(n_tokens >= 0 && max_blocks > 0 && window >= 0, "mixed_attention_mfma: bad sizes");
+    SOMI_REQUIRE(somi_mixed_attention_mfma_supported(heads, kv, dim, vdim, page_size),
+                 "mixed_attention_mfma: %d heads over %d of %d + %d channels in pages of %d are not what the kernel is built for",
+                 heads, kv, dim, vdim, page_size);
+    SOMI_REQUIRE(extra == 0.f || extra == 1.f, "mixed_attention_mfma: the denominator takes 0 or 1 more, got %g", (double)extra);
+    SOMI_REQUIRE(v_pairing == 0 || v_pairing == 1, "mixed_attention_mfma: unknown pairing");
+    if (n_tokens == 0) return 0;
+    const int group = heads / kv;
+    int rp = 1;
+    while (rp < group) rp <<= 1;
+    const int tq = portions ? 16 / rp : 1;
+    const int steps = mxm_steps(dim), accs = mxm_acc(kv, vdim);
+    const size_t lds = mxm_lds_bytes(steps, heads, kv, vdim);
+    const dim3 grid(ceil_div(n_tokens, tq));
+#define MXM_LAUNCH(STEPS, ACC)                                                                                          \
+    do {                                                                                                                \
+        hipError_t err = hipFuncSetAttribute((const void*)mixed_attention_mfma_kernel<STEPS, ACC>,                      \
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
+        if (err != hipSuccess) return somi_fail("mixed_attention_mfma: %s", hipGetErrorString(err));                    \
+        hipLaunchKernelGGL((mixed_attention_mfma_kernel<STEPS, ACC>), grid, dim3(256), lds, stream, (const bf16*)q,     \
+                           (const bf16*)k_cache, (const bf16*)v_cache, block_table, max_blocks, token_entry, positions, \
+                           n_tokens, heads, kv, dim, vdim, page_size, window, scale, cap, extra, talk, v_freq,          \
+                           v_pairing, rp, tq, (bf16*)out);                                                              \
+    } while (0)
+#define MXM_BY_ACC(STEPS)                            \
+    do {                                             \
+        if (accs == 2) MXM_LAUNCH(STEPS, 2);         \
+        else if (accs == 4) MXM_LAUNCH(STEPS, 4);    \
+        else if (accs == 8) MXM_LAUNCH(STEPS, 8);    \
+        else MXM_LAUNCH(STEPS, 16);                  \
+    } while (0)
+    if (steps == 1) MXM_BY_ACC(1);
+    else if (steps == 2) MXM_BY_ACC(2);
+    else if (steps == 4) MXM_BY_ACC(4);
+    else MXM_BY_ACC(8);
+#undef MXM_BY_ACC
+#undef MXM_LAUNCH
+    SOMI_LAUNCH_CHECK("mixed_attention_mfma");
+    return 0;
+}

@@ -1433,8 +1433,8 @@ LATENT_MAX_SPLITS = 64
 
 
 def latent_attention_mfma(queries: torch.Tensor, latent: torch.Tensor, latent_t: torch.Tensor, block_table: torch.Tensor,
-                          token_entry: torch.Tensor, positions: torch.Tensor, rank: int, scale: float, sink: torch.Tensor,
-                          max_context: int, portions: bool = False) -> torch.Tensor:
+                          token_entry: torch.Tensor, positions: torch.Tensor, rank: int, scale: float,
+                          sink: torch.Tensor | None, max_context: int, portions: bool = False, window: int = 0) -> torch.Tensor:
     """:func:`latent_attention_plain` on the matrix cores (bfloat16).  ``latent_t``: [pages, rank, page], the latents
     transposed inside their pages.  ``max_context``: the longest context of the step, known to the host; a step of few
     tokens splits every token's keys over several workgroups, so that the device is busy.  ``portions``: the step holds
@@ -1449,16 +1449,19 @@ def latent_attention_mfma(queries: torch.Tensor, latent: torch.Tensor, latent_t:
     _need(block_table, "block table", torch.int32)
     _need(token_entry, "token entries", torch.int32, (n,))
     _need(positions, "positions", torch.int32, (n,))
-    _need(sink, "sinks", torch.float32, (heads,))
+    if sink is not None:
+        _need(sink, "sinks", torch.float32, (heads,))
     groups = n * ((heads + 15) // 16)
-    tiles = max(1, (int(max_context) + LATENT_SPLIT_KEYS - 1) // LATENT_SPLIT_KEYS)
+    seen = int(max_context) if window <= 0 else min(int(max_context), int(window) + LATENT_SPLIT_KEYS - 1)
+    tiles = max(1, (seen + LATENT_SPLIT_KEYS - 1) // LATENT_SPLIT_KEYS)
     splits = 1 if portions else max(1, min(LATENT_MAX_SPLITS, tiles, (2 * compute_units()) // max(groups, 1)))
     out = torch.empty((n, heads, rank), dtype=torch.bfloat16, device=queries.device)
     part = torch.empty((n * heads * splits * (rank + 2),), dtype=torch.float32, device=queries.device) if splits > 1 else None
     _check(library().somi_latent_attention_mfma(_ptr(queries), _ptr(latent), _ptr(latent_t), _ptr(block_table),
                                                 block_table.shape[1], _ptr(token_entry), _ptr(positions), n, heads,
-                                                int(rank), width - int(rank), latent.shape[1], ctypes.c_float(scale),
-                                                _ptr(sink), splits, 1 if portions else 0, _ptr(out), _ptr(part), _stream()))
+                                                int(rank), width - int(rank), latent.shape[1], int(window),
+                                                ctypes.c_float(scale), _ptr(sink), splits, 1 if portions else 0, _ptr(out),
+                                                _ptr(part), _stream()))
     return out
 
 
@@ -1507,7 +1510,7 @@ def mixed_attention_store(rows: torch.Tensor, positions: torch.Tensor, slots: to
     """From float32 rows [q (heads * dim) | k (kv_heads * dim) | v (kv_heads * vdim)] as projected: q with its first
     ``rot_dims`` channels a head rotated -> [N, heads * dim] in ``out_dtype``; k rotated likewise and v, rotated over all
     its channels with ``value_freq`` ([vdim / 2]) if given, into the tokens' slots of ``k_cache`` [pages, kv_heads, page,
-    dim] and ``v_cache`` [pages, kv_heads, page, vdim].  Without the caches the rows hold q only."""
+    dim] and ``v_cache`` [pages, kv_heads, vdim, page] (transposed inside a page).  Without the caches the rows hold q only."""
     _need(rows, "projected rows", torch.float32)
     n = rows.shape[0]
     _need(positions, "positions", torch.int32, (n,))
@@ -1517,7 +1520,7 @@ def mixed_attention_store(rows: torch.Tensor, positions: torch.Tensor, slots: to
         pages, page = k_cache.shape[0], k_cache.shape[2]
         if tuple(k_cache.shape) != (pages, kv_heads, page, dim):
             raise KernelError(f"mixed_attention_store: key pages {tuple(k_cache.shape)} != [pages, {kv_heads}, page, {dim}]")
-        _need(v_cache, "value pages", out_dtype, (pages, kv_heads, page, vdim))
+        _need(v_cache, "value pages", out_dtype, (pages, kv_heads, vdim, page))
         _need(slots, "slot mapping", torch.int32, (n,))
     if rows.shape[1] != heads * dim + (kv_heads * (dim + vdim) if k_cache is not None else 0):
         raise KernelError(f"mixed_attention_store: rows of {rows.shape[1]} values do not hold the projections")
@@ -1550,9 +1553,9 @@ def mixed_attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
     if q.shape[1] != heads * dim or heads % kv_heads:
         raise KernelError(f"mixed_attention: queries {tuple(q.shape)} do not fit {heads} heads over key pages {tuple(k_cache.shape)}")
     _need(v_cache, "value pages", q.dtype)
-    if v_cache.dim() != 4 or tuple(v_cache.shape[:3]) != (pages, kv_heads, page):
+    if v_cache.dim() != 4 or tuple(v_cache.shape[:2]) != (pages, kv_heads) or v_cache.shape[3] != page:
         raise KernelError(f"mixed_attention: value pages {tuple(v_cache.shape)} do not fit key pages {tuple(k_cache.shape)}")
-    vdim = v_cache.shape[3]
+    vdim = v_cache.shape[2]
     _need(block_table, "block table", torch.int32)
     _need(token_entry, "token entries", torch.int32, (n,))
     _need(positions, "positions", torch.int32, (n,))
@@ -1566,6 +1569,49 @@ def mixed_attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
                                                 kv_heads, dim, vdim, page, int(window), ctypes.c_float(scale),
                                                 ctypes.c_float(softcap), ctypes.c_float(denominator_extra), _ptr(talk),
                                                 _ptr(value_freq), pairing_code(value_pairing), _ptr(out), _stream()))
+    return out
+
+
+def mixed_attention_mfma_supported(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, heads: int) -> bool:
+    """The matrix-core kernel takes these operands: bfloat16, at most 16 query heads a key/value head, key channels a
+    multiple of 8 (up to 256), value channels a multiple of 16, pages of a multiple of 8 tokens, and sizes whose tiles
+    fit a compute unit's LDS."""
+    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16 or q.data_ptr() % 16:
+        return False
+    return bool(library().somi_mixed_attention_mfma_supported(int(heads), k_cache.shape[1], k_cache.shape[3],
+                                                              v_cache.shape[2], k_cache.shape[2]))
+
+
+def mixed_attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                         token_entry: torch.Tensor, positions: torch.Tensor, heads: int, window: int, scale: float,
+                         softcap: float, denominator_extra: float, talk: torch.Tensor | None,
+                         value_freq: torch.Tensor | None, value_pairing: str = "half", portions: bool = False) -> torch.Tensor:
+    """:func:`mixed_attention_plain` on the matrix cores (bfloat16).  ``portions``: the step holds prompt portions, and
+    consecutive tokens share a workgroup (as many as fill 16 query slots a key/value head), so that it reads a tile of
+    keys once for all of them; otherwise a workgroup serves one token."""
+    _need(q, "queries", torch.bfloat16)
+    n = q.shape[0]
+    _need(k_cache, "key pages", torch.bfloat16)
+    pages, kv_heads, page, dim = k_cache.shape
+    if q.shape[1] != heads * dim or heads % kv_heads:
+        raise KernelError(f"mixed_attention: queries {tuple(q.shape)} do not fit {heads} heads over key pages {tuple(k_cache.shape)}")
+    _need(v_cache, "value pages", torch.bfloat16)
+    if v_cache.dim() != 4 or tuple(v_cache.shape[:2]) != (pages, kv_heads) or v_cache.shape[3] != page:
+        raise KernelError(f"mixed_attention: value pages {tuple(v_cache.shape)} do not fit key pages {tuple(k_cache.shape)}")
+    vdim = v_cache.shape[2]
+    _need(block_table, "block table", torch.int32)
+    _need(token_entry, "token entries", torch.int32, (n,))
+    _need(positions, "positions", torch.int32, (n,))
+    if talk is not None:
+        _need(talk, "head mix", torch.float32, (heads, heads))
+    if value_freq is not None:
+        _need(value_freq, "value rotation frequencies", torch.float32, (vdim // 2,))
+    out = torch.empty((n, heads * vdim), dtype=torch.bfloat16, device=q.device)
+    _check(library().somi_mixed_attention_mfma(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+                                               _ptr(token_entry), _ptr(positions), n, int(heads), kv_heads, dim, vdim, page,
+                                               int(window), ctypes.c_float(scale), ctypes.c_float(softcap),
+                                               ctypes.c_float(denominator_extra), _ptr(talk), _ptr(value_freq),
+                                               pairing_code(value_pairing), 1 if portions else 0, _ptr(out), _stream()))
     return out
 
 

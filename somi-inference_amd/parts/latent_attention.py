@@ -148,11 +148,10 @@ class LatentAttention(Mixer):
         """The weighted sums of the kept latents for ``queries`` [N, heads, rank + rot] (the plain part already on the
         latent's side) -> [N, heads, rank].  bfloat16 sizes the matrix-core kernel is built for take it (it reads the
         transposed pages ``latent_t``); float32 and other sizes take the plain kernel."""
-        if (latent_t is not None and self.window is None and self.sink is not None
-                and ops.latent_attention_mfma_supported(queries, latent, self.kv_rank)):
+        if latent_t is not None and ops.latent_attention_mfma_supported(queries, latent, self.kv_rank):
             return ops.latent_attention_mfma(queries, latent, latent_t, view.block_table, step.token_entry, step.positions,
                                              self.kv_rank, self.scale, self.sink, step.max_context,
-                                             portions=step.max_entry_len >= self.PORTION_TOKENS)
+                                             portions=step.max_entry_len >= self.PORTION_TOKENS, window=self.window or 0)
         return ops.latent_attention_plain(queries, latent, view.block_table, step.token_entry, step.positions,
                                           self.kv_rank, self.scale, self.sink, window=self.window or 0)
 

@@ -35,6 +35,7 @@ from .registry import build_part
 
 class MixedHeadsAttention(Mixer):
     graph_safe = True
+    PORTION_TOKENS = 4     # a step whose longest entry has this many tokens runs the kernel with several tokens a workgroup
 
     ROLES = {"q": "q", "k": "k", "v": "v", "o": "o", "talk": "talk", "position": "rotary_emb"}
 
@@ -125,10 +126,12 @@ class MixedHeadsAttention(Mixer):
 
     # -------------------------------------------------------------------- cache
     def cache_spec(self) -> PagedSpec | None:
+        """Keys by token, ``[pages, kv_heads, page, dim]``; values transposed inside a page, ``[pages, kv_heads,
+        value_dim, page]`` (consecutive positions of one channel adjacent: the operand layout of weights times values)."""
         if self.shares_cache:
             return None
         return PagedSpec((PageTensor("k", (self.num_kv_heads, PAGE, self.dim)),
-                          PageTensor("v", (self.num_kv_heads, PAGE, self.value_dim))), self.window)
+                          PageTensor("v", (self.num_kv_heads, self.value_dim, PAGE))), self.window)
 
     # ------------------------------------------------------------------ forward
     def forward(self, x, step, cache: LayerCache | None):
@@ -153,7 +156,14 @@ class MixedHeadsAttention(Mixer):
         return self.out.deferred(attended)
 
     def attend(self, q: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, step, view) -> torch.Tensor:
-        """[N, heads * dim] rotated queries -> [N, heads * value_dim], over the pages of each token's request."""
+        """[N, heads * dim] rotated queries -> [N, heads * value_dim], over the pages of each token's request.  bfloat16
+        sizes the matrix-core kernel is built for take it; float32 and other sizes take the plain kernel."""
+        pairing = (self.value_rotation or {}).get("pairing", "half")
+        if ops.mixed_attention_mfma_supported(q, keys, values, self.num_heads):
+            return ops.mixed_attention_mfma(q, keys, values, view.block_table, step.token_entry, step.positions,
+                                            self.num_heads, self.window or 0, self.scale, self.softcap,
+                                            1.0 if self.sink_one else 0.0, self.talk, self.value_freq, pairing,
+                                            portions=step.max_entry_len >= self.PORTION_TOKENS)
         return ops.mixed_attention_plain(q, keys, values, view.block_table, step.token_entry, step.positions,
                                          self.num_heads, self.window or 0, self.scale, self.softcap,
                                          1.0 if self.sink_one else 0.0, self.talk, self.value_freq,

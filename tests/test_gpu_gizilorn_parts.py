@@ -375,3 +375,41 @@ def test_the_gate_reads_the_mixers_own_input(dtype):
     x = rounded(torch.randn(12, 48, generator=torch.Generator().manual_seed(2)), dtype)
     want = plain.latent_attention(x, w, "m.", m, plain.latent_of(x, w, "m.", m, 1e-6))
     check(PartEngine([part], dtype, DEV, 8).run_cut("a", x, [12])[0], want, dtype)
+
+
+# ------------------------------------------------------------------------------------------ which kernel runs
+def test_which_sizes_take_the_matrix_core_kernels():
+    def pages(kv, dim, vdim, page):
+        return (torch.zeros(4, kv, page, dim, dtype=torch.bfloat16, device=DEV),
+                torch.zeros(4, kv, vdim, page, dtype=torch.bfloat16, device=DEV))
+    q = torch.zeros(2, 8 * 64, dtype=torch.bfloat16, device=DEV)
+    assert ops.mixed_attention_mfma_supported(q, *pages(2, 64, 64, 16), 8)
+    assert ops.mixed_attention_mfma_supported(q, *pages(8, 64, 128, 8), 8)
+    assert not ops.mixed_attention_mfma_supported(q, *pages(2, 64, 24, 16), 8)       # value channels no multiple of 16
+    assert not ops.mixed_attention_mfma_supported(q, *pages(2, 64, 64, 4), 8)        # pages shorter than 8 tokens
+    assert not ops.mixed_attention_mfma_supported(q.float(), *pages(2, 64, 64, 16), 8)
+    q = torch.zeros(2, 34 * 8, dtype=torch.bfloat16, device=DEV)
+    assert not ops.mixed_attention_mfma_supported(q, *pages(2, 8, 16, 16), 34)       # 17 query heads a key/value head
+
+
+@pytest.mark.parametrize("portions", [False, True])
+@pytest.mark.parametrize("heads,kv,dim,vdim,window,cap", [(8, 4, 64, 64, 21, 20.0), (6, 2, 24, 32, None, None),
+                                                          (5, 5, 128, 16, 100, 7.0), (16, 1, 32, 48, 3, None)])
+def test_matrix_core_and_plain_attention_agree(portions, heads, kv, dim, vdim, window, cap):
+    """The two kernels on the same pages, block table and queries: tokens of three requests side by side, one of them
+    with a single token at a high position."""
+    gen = torch.Generator().manual_seed(heads * dim)
+    page, n_pages = 8, 40
+    keys = (torch.randn(n_pages, kv, page, dim, generator=gen) * 0.5).to(torch.bfloat16).to(DEV)
+    values = torch.randn(n_pages, kv, vdim, page, generator=gen).to(torch.bfloat16).to(DEV)
+    table = torch.randperm(n_pages, generator=gen)[:36].view(3, 12).to(torch.int32).to(DEV)
+    lengths = [(0, 37), (60, 9), (90, 1)]                        # (first position, tokens) of the three requests
+    entry = torch.tensor(sum([[e] * n for e, (_, n) in enumerate(lengths)], []), dtype=torch.int32, device=DEV)
+    position = torch.tensor(sum([list(range(p, p + n)) for p, n in lengths], []), dtype=torch.int32, device=DEV)
+    q = torch.randn(entry.numel(), heads * dim, generator=gen).to(torch.bfloat16).to(DEV)
+    talk = (torch.eye(heads) + 0.3 * torch.randn(heads, heads, generator=gen)).to(DEV)
+    freq = (1.0 / (50.0 ** (torch.arange(0, vdim, 2, dtype=torch.float64) / vdim))).float().to(DEV)
+    args = (q, keys, values, table, entry, position, heads, window or 0, dim ** -0.5, cap or 0.0, 1.0, talk, freq, "half")
+    want = ops.mixed_attention_plain(*args)
+    got = ops.mixed_attention_mfma(*args, portions=portions)
+    check(got, want, torch.bfloat16)
