@@ -172,6 +172,62 @@ def metitar_closest_config_dict(sizes: str) -> dict:
             "residual_mult": 0.5, "token_side": {"dim": side}, "layers": [layer] * METITAR_LAYERS}
 
 
+# layer sizes of Gizilorn models that resemble real ones: (width, streams, attention heads, key/value heads, head size,
+# the attention's window, latent-attention heads, unrotated and rotated query/key channels a head, value size, latent
+# size, the latent attention's window, the dense feed-forward's size, vocabulary).  Six layers: latent attention, latent
+# attention that reads the first layer's latent, two attention layers with mixed heads, latent attention, attention.
+GIZILORN_SIZES = {
+    "1b": (2048, 4, 16, 4, 128, 1024, 16, 128, 64, 128, 512, 4096, 4096, 32000),
+    "7b": (4096, 4, 32, 8, 128, 2048, 32, 128, 64, 128, 512, 4096, 8192, 32000),
+}
+GIZILORN_LAYERS = 6
+
+
+def gizilorn_config_dict(sizes: str) -> dict:
+    (width, streams, heads, kv_heads, dim, window, l_heads, l_dim, rot, vdim, rank, l_window, ff, vocab) = GIZILORN_SIZES[sizes]
+    dense = {"kind": "dense", "ff": ff}
+
+    def latent(kv_from=None):
+        mixer = {"heads": l_heads, "dim": l_dim, "rot_dim": rot, "vdim": vdim, "kv_rank": rank, "scale": (l_dim + rot) ** -0.5,
+                 "mask": {"size": l_window}, "rot": {"base": 250000.0, "dims": rot}}
+        if kv_from is not None:
+            mixer["kv_from"] = kv_from
+        return {"type": "latent_attention", "mixer": mixer, "mlp": dense}
+    attention = {"type": "attention", "mlp": dense,
+                 "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "softcap": 30.0,
+                           "mask": {"size": window}, "rot": {"base": 20000.0, "dims": dim}}}
+    return {"architecture": "Gizilorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "streams": streams,
+            "layers": [latent(), latent(0), attention, attention, latent(), attention]}
+
+
+def gizilorn_closest_config_dict(sizes: str) -> dict:
+    """The closest model the engine had before, for the latent attention, the dense feed-forwards and what stands
+    between the sublayers: a Metitar model of six latent-attention layers of the same width, heads, head sizes and
+    latent (with a query latent of three quarters of the width's half, a sink, and no window: it is causal over
+    everything) and dense feed-forwards of the same size; no input convolution, no token input."""
+    (width, streams, heads, kv_heads, dim, window, l_heads, l_dim, rot, vdim, rank, l_window, ff, vocab) = GIZILORN_SIZES[sizes]
+
+    def latent(kv_from=None):
+        mixer = {"heads": l_heads, "dim": l_dim, "rot_dim": rot, "vdim": vdim, "kv_rank": rank, "q_rank": 3 * width // 8,
+                 "scale": (l_dim + rot) ** -0.5, "rot": {"base": 10000.0, "dims": rot}}
+        if kv_from is not None:
+            mixer["kv_from"] = kv_from
+        return {"type": "latent_attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff}}
+    return {"architecture": "Metitar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+            "logit_scale": 1.0, "layers": [latent(), latent(0), latent(), latent(), latent(), latent(4)]}
+
+
+def gizilorn_closest_attention_config_dict(sizes: str) -> dict:
+    """The closest model for the attention with mixed heads: a Qwen2.5-style model of the same width, heads, key/value
+    heads, head size and window in every layer."""
+    (width, streams, heads, kv_heads, dim, window, l_heads, l_dim, rot, vdim, rank, l_window, ff, vocab) = GIZILORN_SIZES[sizes]
+    return {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "vocab_size": vocab, "hidden_size": width,
+            "intermediate_size": ff, "num_hidden_layers": GIZILORN_LAYERS, "num_attention_heads": heads,
+            "num_key_value_heads": kv_heads, "head_dim": dim, "rope_theta": 2e4, "rms_norm_eps": 1e-6,
+            "tie_word_embeddings": False, "max_position_embeddings": 32768, "hidden_act": "silu", "attention_bias": True,
+            "use_sliding_window": True, "sliding_window": window, "max_window_layers": 0}
+
+
 # keys of a config.json that name sizes, in the order they are reported under "config" (flat, at most 20 keys)
 SIZE_KEYS = ("hidden_size", "intermediate_size", "num_attention_heads", "num_key_value_heads", "head_dim",
              "vocab_size", "tie_word_embeddings")
@@ -216,6 +272,11 @@ def parse_args() -> argparse.Namespace:
                    help="instead of the default workload: prefill and decode of a Metitar model (attention over a shared "
                         "latent, the HGRN2 recurrence, dense and routed feed-forwards) at these layer sizes, beside the "
                         "Rusolorn model of equal width, heads, experts and layers, each with its stage times")
+    p.add_argument("--gizilorn", default=None, choices=sorted(GIZILORN_SIZES), metavar="SIZES",
+                   help="instead of the default workload: prefill and decode of a Gizilorn model (several residual "
+                        "streams, attention with mixed heads, windowed attention over a shared latent) at these layer "
+                        "sizes, beside a Metitar model of equal width, latent and feed-forwards and a Qwen2.5-style model "
+                        "of equal width, heads and window, each with its stage times")
     p.add_argument("--serving", type=int, default=0, metavar="REQUESTS",
                    help="also run this many requests (prompts of 128 to 2,048 tokens, 256 new tokens each) through "
                         "the scheduler with portions of 512, and report it under 'serving'")
@@ -782,6 +843,81 @@ def run_metitar(args) -> dict:
     return out
 
 
+def run_gizilorn(args) -> dict:
+    """Prefill and decode of a Gizilorn model beside the closest models the engine had, with the stage times of all
+    three and what the attention kernels, the dense products and the kernels between the sublayers reach of the machine."""
+    (width, streams, heads, kv_heads, dim, window, l_heads, l_dim, rot, vdim, rank, l_window, ff, vocab) = GIZILORN_SIZES[args.gizilorn]
+    batches, context, tokens = (8, 64), args.context, args.prefill_tokens
+    out: dict = {}
+    for label, config_dict in (("gizilorn", gizilorn_config_dict(args.gizilorn)),
+                               ("closest", gizilorn_closest_config_dict(args.gizilorn)),
+                               ("closest_attention", gizilorn_closest_attention_config_dict(args.gizilorn))):
+        bench = Workbench(config_dict, dtype=args.dtype, seed=args.seed, block_size=args.block_size,
+                          pool_tokens=Workbench.pool_tokens(batches, context, tokens), max_requests=max(batches))
+        block: dict = {"prefill": {str(n): bench.prefill_run(n) for n in sorted({512, tokens})}}
+        for batch in batches:
+            run = bench.decode_run(batch, max(POINT_MIN_STEPS, args.steps // 2), max(2, args.warmup // 2), context)
+            block[f"decode_b{batch}"] = {"tok_s": round(run["tok_s"], 1), "ms": round(run["ms"], 4),
+                                        "mean_ctx": round(run["mean_ctx"], 1)}
+        block["stages"] = bench.stage_run(tokens, batches[0], context)
+        print_stage_tables(block["stages"])
+        out[label] = block
+        bench.close()
+    bf16_peak = PEAK_FLOPS["bfloat16"]
+
+    def pairs_of(size):
+        return sum(min(p + 1, size) for p in range(tokens))
+
+    def stage_ms(block, run, *names):
+        return sum(block["stages"][run].get(name, {}).get("ms", 0.0) for name in names)
+
+    def rate(flops, ms):
+        return {"ms": round(ms, 4), "tflops": round(flops / 1e9 / max(ms, 1e-9), 2),
+                "frac_of_peak": round(flops / 1e3 / max(ms, 1e-9) / bf16_peak * 1e6, 5)}
+
+    def stream(bytes_, ms):
+        return {"ms": round(ms, 4), "gbs": round(bytes_ / 1e6 / max(ms, 1e-9), 1)}
+    run, layers, half = f"prefill_{tokens}", GIZILORN_LAYERS, GIZILORN_LAYERS // 2
+    out["prefill_kernels"] = {
+        "tokens": tokens,
+        # useful work over the visible pairs: scores once and weights times values once (the kernel computes the scores
+        # twice, mixes the heads' weights and multiplies the weights in two halves)
+        "gizilorn_attention": rate(half * 2.0 * heads * (dim + dim) * pairs_of(window),
+                                   stage_ms(out["gizilorn"], run, "mixed attention")),
+        "closest_attention": rate(layers * 4.0 * heads * dim * pairs_of(window), stage_ms(out["closest_attention"], run, "attention")),
+        "closest_latent_attention": rate(layers * 2.0 * l_heads * (2 * rank + rot) * pairs_of(tokens),
+                                         stage_ms(out["closest"], run, "attention")),
+        "gizilorn_dense": rate(layers * 4.0 * tokens * ff * width, stage_ms(out["gizilorn"], run, "up", "down")),
+        "closest_dense": rate(layers * 4.0 * tokens * ff * width, stage_ms(out["closest"], run, "up", "down")),
+        # between the sublayers: every stream read and written in float32, the sublayer's rows read, the normed rows written
+        "gizilorn_streams": stream(layers * 2.0 * tokens * width * (8.0 * streams + 4 + 2),
+                                   stage_ms(out["gizilorn"], run, "residual add, norm")),
+        "closest_output_norm": stream(layers * 2.0 * tokens * width * (8.0 + 4 + 2),
+                                      stage_ms(out["closest"], run, "output norm, residual add")),
+    }
+    run = f"decode_b{batches[0]}_eager"
+    out["decode_kernels"] = {
+        "batch": batches[0], "context": context,
+        "gizilorn_attention": stream(half * batches[0] * min(context, window) * kv_heads * 2 * dim * 2.0,
+                                     stage_ms(out["gizilorn"], run, "mixed attention")),
+        "closest_attention": stream(layers * batches[0] * min(context, window) * kv_heads * 2 * dim * 2.0,
+                                    stage_ms(out["closest_attention"], run, "attention")),
+        "closest_latent_attention": stream(layers * batches[0] * context * (rank + rot) * 2.0,
+                                           stage_ms(out["closest"], run, "attention")),
+        "gizilorn_streams": stream(layers * 2.0 * batches[0] * width * (8.0 * streams + 4 + 2),
+                                   stage_ms(out["gizilorn"], run, "residual add, norm")),
+    }
+    for kernels, tokens_or_batch, seen in ((out["prefill_kernels"], None, pairs_of(l_window)),
+                                           (out["decode_kernels"], batches[0], None)):
+        name = "prefill_%d" % tokens if tokens_or_batch is None else run
+        ms = stage_ms(out["gizilorn"], name, "attention")
+        if tokens_or_batch is None:
+            kernels["gizilorn_latent_attention"] = rate(half * 2.0 * l_heads * (2 * rank + rot) * seen, ms)
+        else:
+            kernels["gizilorn_latent_attention"] = stream(half * tokens_or_batch * min(context, l_window) * (rank + rot) * 2.0, ms)
+    return out
+
+
 def main() -> int:
     args = parse_args()
     world = int(os.environ.get("WORLD_SIZE", "1"))
@@ -796,6 +932,16 @@ def main() -> int:
                 "data": "synthetic: seeded random weights, seeded uniform token ids", "sizes": args.kamedra}
         line.update(run_kamedra(args))
         line["value"] = line["kamedra"][f"decode_b8"]["tok_s"]
+        line["seconds_total"] = round(time.perf_counter() - started, 1)
+        print(json.dumps(line))
+        return 0
+
+    if args.gizilorn:
+        line = {"metric": f"Gizilorn at {args.gizilorn} layer sizes beside the closest Metitar and Qwen2.5-style models: prefill and decode",
+                "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                "data": "synthetic: seeded random weights, seeded uniform token ids", "sizes": args.gizilorn}
+        line.update(run_gizilorn(args))
+        line["value"] = line["gizilorn"]["decode_b8"]["tok_s"]
         line["seconds_total"] = round(time.perf_counter() - started, 1)
         print(json.dumps(line))
         return 0

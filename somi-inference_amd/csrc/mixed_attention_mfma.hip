@@ -9,11 +9,12 @@
 //   first walk   wavefront w takes the key/value heads w, w + 4, ...; 16 keys at a time, S^T = K Q^T by `16x16x32`
 //                products (K fragments straight from the pages, Q fragments from LDS); a lane holds 4 keys of one slot
 //                and keeps a running maximum and sum of its own, joined over the lanes at the end: (m, l) of every slot
-//   second walk  32 keys at a time: the same scores again, p = exp(s - m) / l in float32 into LDS; then all threads mix,
-//                w_h = sum_g T[h, g] p_g, float32, and leave the mixed weights in LDS as two bfloat16 halves (w = hi + lo,
-//                so no weight is rounded to eight bits); then O^T = V^T W^T, the V^T fragments straight from the pages
-//                (values are stored transposed inside a page), each wavefront owning some (key/value head, 16 channels)
-//                tiles of the output
+//   second walk  32 keys at a time: the same scores again, p = exp(s - m) / l in float32, which goes to LDS by (token,
+//                key) and head as two bfloat16 halves (p = hi + lo, so no weight is rounded to eight bits); the mix W^T =
+//                P^T T^T as matrix products too (T in two halves as well: hi hi + lo hi + hi lo), whose results go to LDS
+//                by key/value head and slot, again in two halves; then O^T = V^T W^T, the V^T fragments straight from
+//                the pages (values are stored transposed inside a page), each wavefront owning some (key/value head, 16
+//                channels) tiles of the output
 //   end          the sums go through LDS, are turned back by the query's position where values were turned by theirs,
 //                and are written out
 //
@@ -24,13 +25,18 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 mxm_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float mxm_f32x4;
 
-#define MXM_PROW 33            // floats a slot's 32 weights take in LDS (one more: slots fall on different banks)
-#define MXM_WROW 40            // bfloat16 a slot's 32 mixed weights take (rows stay 16-byte aligned)
+#define MXM_WROW 40            // bfloat16 a row of 32 weights takes in LDS (rows stay 16-byte aligned)
 
+// cap * tanh(s / cap) with tanh(x) = 1 - 2 / (1 + exp(2 x)): float32, a handful of instructions
 __device__ __forceinline__ float mxm_cap(float s, float cap, float inv_cap) {
-    return cap > 0.f ? cap * tanhf(s * inv_cap) : s;
+    return cap > 0.f ? cap * (1.0f - 2.0f / (1.0f + __expf(2.0f * s * inv_cap))) : s;
 }
 
+// mode 0: a workgroup walks all keys of its tokens and writes their outputs.  Modes 1 and 2 split a token's keys over
+// `gridDim.y` workgroups (one token a workgroup): mode 1 leaves every head's (maximum, sum) over the split's keys in
+// `stats` [tokens, splits, heads, 2]; mode 2 joins the splits' statistics itself (with the sink's share), forms the
+// weights of its keys against the joined maximum and sum, and leaves its unnormed share of the output, which is simply a
+// term of the sum over the splits, in `part` [tokens, splits, heads * vdim] (not yet turned back).
 template <int STEPS, int ACC>
 __global__ void __launch_bounds__(256)
 mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
@@ -38,21 +44,26 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
                             const int* __restrict__ positions, int n_tokens, int heads, int kv, int dim, int vdim,
                             int page_size, int window, float scale, float cap, float extra,
                             const float* __restrict__ talk, const float* __restrict__ v_freq, int v_pairing, int rp,
-                            int tq, bf16* __restrict__ out) {
+                            int tq, int mode, float* __restrict__ stats, float* __restrict__ part,
+                            bf16* __restrict__ out) {
     constexpr int QROW = STEPS * 32 + 8;
+    const int hp = (heads + 31) & ~31, trow = hp + 8;       // heads padded to the products' K, and a row of them in LDS
     extern __shared__ __attribute__((aligned(16))) char mxm_lds[];
     bf16* q_s = reinterpret_cast<bf16*>(mxm_lds);                                  // [kv][16][QROW]
-    float* ml = reinterpret_cast<float*>(q_s + (size_t)kv * 16 * QROW);            // [kv][16][2]
-    float* P = ml + (size_t)kv * 32;                                               // [kv][16][PROW]
-    float* talk_s = P + (size_t)kv * 16 * MXM_PROW;                                // [heads][heads]
-    bf16* w_hi = reinterpret_cast<bf16*>(talk_s + ((heads * heads + 3) & ~3));     // [kv][16][WROW]
+    bf16* t_hi = q_s + (size_t)kv * 16 * QROW;                                     // [hp (to)][trow (from)]
+    bf16* t_lo = t_hi + (size_t)hp * trow;
+    bf16* p_hi = t_lo + (size_t)hp * trow;                                         // [tq * 32 (token, key)][trow (head)]
+    bf16* p_lo = p_hi + (size_t)tq * 32 * trow;
+    bf16* w_hi = p_lo + (size_t)tq * 32 * trow;                                    // [kv][16][WROW]
     bf16* w_lo = w_hi + (size_t)kv * 16 * MXM_WROW;
+    float* ml = reinterpret_cast<float*>(w_lo + (size_t)kv * 16 * MXM_WROW);       // [kv][16][2]
     float* o_s = reinterpret_cast<float*>(mxm_lds);                                // [kv][16][vdim], over all of the above
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, col = lane & 15, quad = lane >> 4;
     const int group = heads / kv, dts = vdim >> 4;
     const int t0 = (int)blockIdx.x * tq;
     const int count = min(tq, n_tokens - t0);
+    const int split = blockIdx.y, splits = gridDim.y;
     const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
     const int my_u = col / rp, my_r = col % rp;          // the token and head-in-group of the slot this lane serves
 
@@ -61,16 +72,28 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
         int r1 = r0 + 1;
         while (r1 < count && token_entry[t0 + r1] == entry) ++r1;
         const int* table = block_table + (int64_t)entry * max_blocks;
-        const int p_first = positions[t0 + r0], k_hi = positions[t0 + r1 - 1];
+        const int p_first = positions[t0 + r0], p_last = positions[t0 + r1 - 1];
         const int k_lo = window > 0 ? max(0, p_first - window + 1) : 0;
-        const int kb0 = k_lo & ~31;
+        // this workgroup's keys: whole 32-key chunks (aligned to absolute positions) of k_lo .. p_last
+        const int chunks = ((p_last - (k_lo & ~31)) >> 5) + 1, per = (chunks + splits - 1) / splits;
+        const int kb0 = (k_lo & ~31) + split * per * 32;
+        const int k_hi = min(p_last, kb0 + per * 32 - 1);
         const bool live = my_u >= r0 && my_u < r1 && my_r < group;
         const int my_pos = live ? positions[t0 + my_u] : -1;
         const int my_first = window > 0 ? max(0, my_pos - window + 1) : 0;
 
-        // ---- the mix (the end of a run writes over it) and the queries of the run's tokens, slot by slot
-        for (int i = tid; i < heads * heads; i += 256)
-            talk_s[i] = talk != nullptr ? talk[i] : (i / heads == i % heads ? 1.f : 0.f);
+        // ---- into LDS (the end of a run writes over all of it): the mix in two bfloat16 halves, zeros where weights
+        //      of dead slots and padded heads would stand, and the queries of the run's tokens, slot by slot
+        for (int i = tid; i < hp * trow; i += 256) {
+            const int h = i / trow, g = i % trow;
+            float t = 0.f;
+            if (h < heads && g < heads) t = talk != nullptr ? talk[h * heads + g] : (h == g ? 1.f : 0.f);
+            const bf16 hi = (bf16)t;
+            t_hi[i] = hi;
+            t_lo[i] = (bf16)(t - (float)hi);
+        }
+        for (int i = tid; i < tq * 32 * trow; i += 256) p_hi[i] = p_lo[i] = (bf16)0.f;
+        for (int i = tid; i < kv * 16 * MXM_WROW; i += 256) w_hi[i] = w_lo[i] = (bf16)0.f;
         for (int i = tid; i < kv * 16 * STEPS * 4; i += 256) {
             const int ch = (i % (STEPS * 4)) * 8, slot = (i / (STEPS * 4)) % 16, c = i / (STEPS * 4 * 16);
             const int u = slot / rp, r = slot % rp;
@@ -85,7 +108,7 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
 
         // scores of 16 keys from kb on against the 16 slots of key/value head c: the lane's 4 keys of its slot
         auto scores = [&](int c, int kb, float (&s4)[4]) {
-            const int key_row = min(kb + col, k_hi);
+            const int key_row = min(kb + col, p_last);
             const int64_t page = table[key_row / page_size];
             const bf16* krow = k_cache + ((page * kv + c) * page_size + key_row % page_size) * dim;
             const bf16* q_lane = q_s + ((size_t)c * 16 + col) * QROW + quad * 8;
@@ -102,36 +125,61 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int key = kb + quad * 4 + i;
-                s4[i] = live && key >= my_first && key <= my_pos ? mxm_cap(sc[i] * scale, cap, inv_cap) : -INFINITY;
+                s4[i] = live && key >= my_first && key <= my_pos && key <= k_hi ? mxm_cap(sc[i] * scale, cap, inv_cap) : -INFINITY;
             }
         };
 
-        // ---- first walk: every slot's maximum and sum
+        // ---- first walk: every slot's maximum and sum (mode 2: joined from what the splits left)
         for (int c = w; c < kv; c += 4) {
             float m = -INFINITY, l = 0.f;
-            for (int kb = kb0; kb <= k_hi; kb += 16) {
-                float s4[4];
-                scores(c, kb, s4);
-                const float mx = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
-                const float m_new = fmaxf(m, mx);
-                if (m_new > -INFINITY) {
-                    l = l * __expf(m - m_new) + ((__expf(s4[0] - m_new) + __expf(s4[1] - m_new)) +
-                                                (__expf(s4[2] - m_new) + __expf(s4[3] - m_new)));
-                    m = m_new;
+            if (mode != 2) {
+                for (int kb = kb0; kb <= k_hi; kb += 16) {
+                    float s4[4];
+                    scores(c, kb, s4);
+                    const float mx = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
+                    const float m_new = fmaxf(m, mx);
+                    if (m_new > -INFINITY) {
+                        l = l * __expf(m - m_new) + ((__expf(s4[0] - m_new) + __expf(s4[1] - m_new)) +
+                                                    (__expf(s4[2] - m_new) + __expf(s4[3] - m_new)));
+                        m = m_new;
+                    }
+                }
+            } else if (live && quad == 0) {
+                const float* mine = stats + (((int64_t)(t0 + my_u) * splits) * heads + c * group + my_r) * 2;
+                for (int s = 0; s < splits; ++s) {
+                    const float m_s = mine[(int64_t)s * heads * 2], l_s = mine[(int64_t)s * heads * 2 + 1];
+                    const float m_new = fmaxf(m, m_s);
+                    if (m_new > -INFINITY) {
+                        l = l * __expf(m - m_new) + l_s * __expf(m_s - m_new);
+                        m = m_new;
+                    }
                 }
             }
             // the four lanes of a slot, then the sink's share
             float top = fmaxf(m, __shfl_xor(m, 16, 64));
             top = fmaxf(top, __shfl_xor(top, 32, 64));
-            if (extra > 0.f) top = fmaxf(top, 0.f);
-            float part = top > -INFINITY ? l * __expf(m - top) : 0.f;
-            part += __shfl_xor(part, 16, 64);
-            part += __shfl_xor(part, 32, 64);
-            if (extra > 0.f) part += extra * __expf(-top);
+            if (extra > 0.f && mode != 1) top = fmaxf(top, 0.f);
+            float sum = top > -INFINITY ? l * __expf(m - top) : 0.f;
+            sum += __shfl_xor(sum, 16, 64);
+            sum += __shfl_xor(sum, 32, 64);
+            if (extra > 0.f && mode != 1) sum += extra * __expf(-top);
             if (quad == 0) {
-                ml[(c * 16 + col) * 2] = top;
-                ml[(c * 16 + col) * 2 + 1] = part;
+                if (mode == 1) {
+                    if (live) {
+                        float* mine = stats + ((((int64_t)(t0 + my_u) * splits + split) * heads) + c * group + my_r) * 2;
+                        mine[0] = top;
+                        mine[1] = sum;
+                    }
+                } else {
+                    ml[(c * 16 + col) * 2] = top;
+                    ml[(c * 16 + col) * 2 + 1] = sum;
+                }
             }
+        }
+        if (mode == 1) {
+            __syncthreads();
+            r0 = r1;
+            continue;
         }
         __syncthreads();
 
@@ -140,36 +188,61 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
 #pragma unroll
         for (int a = 0; a < ACC; ++a) acc[a] = mxm_f32x4{0.f, 0.f, 0.f, 0.f};
         for (int kb = kb0; kb <= k_hi; kb += 32) {
+            // the weights p = exp(s - m) / l, by (token, key) and head, in two bfloat16 halves
             for (int c = w; c < kv; c += 4) {
                 const float m = ml[(c * 16 + col) * 2], inv_l = live ? 1.0f / ml[(c * 16 + col) * 2 + 1] : 0.f;
+                // every lane takes part in the scores (its key row is one of the tile's 16, whatever its slot is)
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
                     float s4[4];
                     scores(c, kb + half * 16, s4);
+                    if (live) {
 #pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        P[((size_t)c * 16 + col) * MXM_PROW + half * 16 + quad * 4 + i] = live ? __expf(s4[i] - m) * inv_l : 0.f;
+                        for (int i = 0; i < 4; ++i) {
+                            const float pv = __expf(s4[i] - m) * inv_l;
+                            const bf16 hi = (bf16)pv;
+                            const size_t at = ((size_t)my_u * 32 + half * 16 + quad * 4 + i) * trow + c * group + my_r;
+                            p_hi[at] = hi;
+                            p_lo[at] = (bf16)(pv - (float)hi);
+                        }
+                    }
                 }
             }
             __syncthreads();
-            for (int i = tid; i < kv * 16 * 32; i += 256) {
-                const int j = i & 31, slot = (i >> 5) & 15, c = i >> 9;
-                const int u = slot / rp, r = slot % rp;
-                float mixed = 0.f;
-                if (u >= r0 && u < r1 && r < group) {
-                    const float* t_row = talk_s + (c * group + r) * heads;
-                    for (int cg = 0; cg < kv; ++cg) {
-                        const float* p_row = P + ((size_t)cg * 16 + u * rp) * MXM_PROW + j;
-                        for (int rg = 0; rg < group; ++rg) mixed = fmaf(t_row[cg * group + rg], p_row[rg * MXM_PROW], mixed);
+            // the mix: W^T [(token, key) x head] = P^T [(token, key) x head] T^T, tiles of 16 x 16 over the wavefronts
+            {
+                const int n_tiles = tq * 2, h_tiles = (heads + 15) >> 4;
+                for (int tile = w; tile < n_tiles * h_tiles; tile += 4) {
+                    const int nt = tile / h_tiles, ht = tile % h_tiles;
+                    mxm_f32x4 mixed = mxm_f32x4{0.f, 0.f, 0.f, 0.f};
+                    for (int ks = 0; ks < hp; ks += 32) {
+                        const size_t pa = ((size_t)nt * 16 + col) * trow + ks + quad * 8;
+                        const size_t ta = ((size_t)ht * 16 + col) * trow + ks + quad * 8;
+                        const mxm_bf16x8 ph = *reinterpret_cast<const mxm_bf16x8*>(p_hi + pa);
+                        const mxm_bf16x8 pl = *reinterpret_cast<const mxm_bf16x8*>(p_lo + pa);
+                        const mxm_bf16x8 th = *reinterpret_cast<const mxm_bf16x8*>(t_hi + ta);
+                        const mxm_bf16x8 tl = *reinterpret_cast<const mxm_bf16x8*>(t_lo + ta);
+                        mixed = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph, th, mixed, 0, 0, 0);
+                        mixed = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl, th, mixed, 0, 0, 0);
+                        mixed = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph, tl, mixed, 0, 0, 0);
+                    }
+                    // the lane holds head ht * 16 + col for the (token, key) pairs nt * 16 + quad * 4 + i
+                    const int h = ht * 16 + col;
+                    if (h < heads) {
+                        const int u = nt >> 1, c = h / group, r = h % group;
+                        const size_t at = ((size_t)c * 16 + u * rp + r) * MXM_WROW + (nt & 1) * 16 + quad * 4;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const bf16 hi = (bf16)mixed[i];
+                            w_hi[at + i] = hi;
+                            w_lo[at + i] = (bf16)(mixed[i] - (float)hi);
+                        }
                     }
                 }
-                const bf16 hi = (bf16)mixed;
-                w_hi[((size_t)c * 16 + slot) * MXM_WROW + j] = hi;
-                w_lo[((size_t)c * 16 + slot) * MXM_WROW + j] = (bf16)(mixed - (float)hi);
             }
             __syncthreads();
             // the lane's 8 keys lie in one page (pages hold a multiple of 8 tokens, the walk is aligned to 32)
-            const int key8 = min(kb + quad * 8, k_hi & ~7);
+            const int key8 = min(kb + quad * 8, p_last & ~7);
             const int64_t page = table[key8 / page_size];
             const int off = key8 % page_size;
 #pragma unroll
@@ -185,7 +258,7 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
                 }
             }
         }
-        // ---- the heads' outputs through LDS, turned back by the query's position
+        // ---- the heads' outputs through LDS, turned back by the query's position (mode 2: the split's share as it is)
         __syncthreads();
 #pragma unroll
         for (int a = 0; a < ACC; ++a) {
@@ -203,6 +276,10 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
             if (u < r0 || u >= r1 || r >= group) continue;
             const float* row = o_s + ((size_t)c * 16 + slot) * vdim;
             float v = row[d];
+            if (mode == 2) {
+                part[(((int64_t)(t0 + u) * splits + split) * heads + c * group + r) * vdim + d] = v;
+                continue;
+            }
             if (v_freq != nullptr) {
                 const int half = vdim >> 1;
                 const bool first = v_pairing == 0 ? d < half : (d & 1) == 0;
@@ -219,9 +296,39 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
     }
 }
 
-static size_t mxm_lds_bytes(int steps, int heads, int kv, int vdim) {
-    const size_t walk = (size_t)kv * 16 * (steps * 32 + 8) * 2 + (size_t)kv * 32 * 4 + (size_t)kv * 16 * MXM_PROW * 4 +
-                        (size_t)((heads * heads + 3) & ~3) * 4 + (size_t)kv * 16 * MXM_WROW * 2 * 2;
+// out[t, h, :] = the sum of the splits' shares, turned back by the token's position.  A thread per (token, head, channel).
+__global__ void __launch_bounds__(256)
+mixed_attention_join_kernel(const float* __restrict__ part, int splits, int heads, int vdim, const int* __restrict__ positions,
+                            const float* __restrict__ v_freq, int v_pairing, bf16* __restrict__ out, int64_t count) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    const int d = (int)(i % vdim);
+    const int64_t th = i / vdim;
+    const int h = (int)(th % heads);
+    const int64_t t = th / heads;
+    const float* mine = part + ((t * splits) * heads + h) * vdim;
+    auto total = [&](int ch) {
+        float sum = 0.f;
+        for (int s = 0; s < splits; ++s) sum += mine[(int64_t)s * heads * vdim + ch];
+        return sum;
+    };
+    float v = total(d);
+    if (v_freq != nullptr) {
+        const int half = vdim >> 1;
+        const bool first = v_pairing == 0 ? d < half : (d & 1) == 0;
+        const int pair = v_pairing == 0 ? (first ? d : d - half) : d >> 1;
+        const float other = total(v_pairing == 0 ? (first ? d + half : d - half) : (d ^ 1));
+        const float angle = (float)positions[t] * v_freq[pair];
+        const float cs = cosf(angle), sn = sinf(angle);
+        v = first ? v * cs + other * sn : v * cs - other * sn;
+    }
+    out[i] = (bf16)v;
+}
+
+static size_t mxm_lds_bytes(int steps, int heads, int kv, int vdim, int tq) {
+    const size_t hp = (size_t)((heads + 31) & ~31), trow = hp + 8;
+    const size_t walk = (size_t)kv * 16 * (steps * 32 + 8) * 2 + 2 * hp * trow * 2 + 2 * (size_t)tq * 32 * trow * 2 +
+                        2 * (size_t)kv * 16 * MXM_WROW * 2 + (size_t)kv * 32 * 4;
     const size_t end = (size_t)kv * 16 * vdim * 4;
     return walk > end ? walk : end;
 }
@@ -237,53 +344,78 @@ extern "C" int somi_mixed_attention_mfma_supported(int heads, int kv, int dim, i
         vdim % 16 || page_size <= 0 || page_size % 8)
         return 0;
     if (ceil_div(kv * (vdim / 16), 4) > 16) return 0;
-    return mxm_lds_bytes(mxm_steps(dim), heads, kv, vdim) <= 160 * 1024 ? 1 : 0;
+    int rp = 1;
+    while (rp < heads / kv) rp <<= 1;
+    return mxm_lds_bytes(mxm_steps(dim), heads, kv, vdim, 16 / rp) <= 160 * 1024 ? 1 : 0;
 }
 
 // As somi_mixed_attention_plain, bfloat16 only.  portions != 0: the step holds prompt portions, and as many consecutive
-// tokens share a workgroup as their heads fill 16 query slots a key/value head; otherwise a workgroup serves one token.
+// tokens share a workgroup as their heads fill 16 query slots a key/value head; otherwise a workgroup serves one token,
+// and with splits > 1 a token's keys are dealt out to that many workgroups (three launches: the splits' statistics,
+// their shares of the output, the join), for which `stats` holds n_tokens * splits * heads * 2 floats and `part`
+// n_tokens * splits * heads * vdim.
 extern "C" int somi_mixed_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int* block_table,
                                          int max_blocks, const int* token_entry, const int* positions, int n_tokens,
                                          int heads, int kv, int dim, int vdim, int page_size, int window, float scale,
                                          float cap, float extra, const float* talk, const float* v_freq, int v_pairing,
-                                         int portions, void* out, hipStream_t stream) {
-    SOMI_REQUIRE(n_tokens >= 0 && max_blocks > 0 && window >= 0, "mixed_attention_mfma: bad sizes");
+                                         int portions, int splits, float* stats, float* part, void* out,
+                                         hipStream_t stream) {
+    SOMI_REQUIRE(n_tokens >= 0 && max_blocks > 0 && window >= 0 && splits >= 1 && splits <= 65535, "mixed_attention_mfma: bad sizes");
     SOMI_REQUIRE(somi_mixed_attention_mfma_supported(heads, kv, dim, vdim, page_size),
                  "mixed_attention_mfma: %d heads over %d of %d + %d channels in pages of %d are not what the kernel is built for",
                  heads, kv, dim, vdim, page_size);
     SOMI_REQUIRE(extra == 0.f || extra == 1.f, "mixed_attention_mfma: the denominator takes 0 or 1 more, got %g", (double)extra);
     SOMI_REQUIRE(v_pairing == 0 || v_pairing == 1, "mixed_attention_mfma: unknown pairing");
+    SOMI_REQUIRE(splits == 1 || (!portions && stats != nullptr && part != nullptr),
+                 "mixed_attention_mfma: key splits are for steps of single tokens and need their workspaces");
     if (n_tokens == 0) return 0;
     const int group = heads / kv;
     int rp = 1;
     while (rp < group) rp <<= 1;
     const int tq = portions ? 16 / rp : 1;
     const int steps = mxm_steps(dim), accs = mxm_acc(kv, vdim);
-    const size_t lds = mxm_lds_bytes(steps, heads, kv, vdim);
-    const dim3 grid(ceil_div(n_tokens, tq));
-#define MXM_LAUNCH(STEPS, ACC)                                                                                          \
+    const size_t lds = mxm_lds_bytes(steps, heads, kv, vdim, tq);
+#define MXM_LAUNCH(STEPS, ACC, MODE, GRID)                                                                              \
     do {                                                                                                                \
         hipError_t err = hipFuncSetAttribute((const void*)mixed_attention_mfma_kernel<STEPS, ACC>,                      \
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
         if (err != hipSuccess) return somi_fail("mixed_attention_mfma: %s", hipGetErrorString(err));                    \
-        hipLaunchKernelGGL((mixed_attention_mfma_kernel<STEPS, ACC>), grid, dim3(256), lds, stream, (const bf16*)q,     \
+        hipLaunchKernelGGL((mixed_attention_mfma_kernel<STEPS, ACC>), GRID, dim3(256), lds, stream, (const bf16*)q,     \
                            (const bf16*)k_cache, (const bf16*)v_cache, block_table, max_blocks, token_entry, positions, \
                            n_tokens, heads, kv, dim, vdim, page_size, window, scale, cap, extra, talk, v_freq,          \
-                           v_pairing, rp, tq, (bf16*)out);                                                              \
+                           v_pairing, rp, tq, MODE, stats, part, (bf16*)out);                                           \
     } while (0)
-#define MXM_BY_ACC(STEPS)                            \
-    do {                                             \
-        if (accs == 2) MXM_LAUNCH(STEPS, 2);         \
-        else if (accs == 4) MXM_LAUNCH(STEPS, 4);    \
-        else if (accs == 8) MXM_LAUNCH(STEPS, 8);    \
-        else MXM_LAUNCH(STEPS, 16);                  \
+#define MXM_BY_ACC(STEPS, MODE, GRID)                            \
+    do {                                                         \
+        if (accs == 2) MXM_LAUNCH(STEPS, 2, MODE, GRID);         \
+        else if (accs == 4) MXM_LAUNCH(STEPS, 4, MODE, GRID);    \
+        else if (accs == 8) MXM_LAUNCH(STEPS, 8, MODE, GRID);    \
+        else MXM_LAUNCH(STEPS, 16, MODE, GRID);                  \
     } while (0)
-    if (steps == 1) MXM_BY_ACC(1);
-    else if (steps == 2) MXM_BY_ACC(2);
-    else if (steps == 4) MXM_BY_ACC(4);
-    else MXM_BY_ACC(8);
+#define MXM_BY_STEPS(MODE, GRID)                         \
+    do {                                                 \
+        if (steps == 1) MXM_BY_ACC(1, MODE, GRID);       \
+        else if (steps == 2) MXM_BY_ACC(2, MODE, GRID);  \
+        else if (steps == 4) MXM_BY_ACC(4, MODE, GRID);  \
+        else MXM_BY_ACC(8, MODE, GRID);                  \
+    } while (0)
+    if (splits == 1) {
+        const dim3 grid(ceil_div(n_tokens, tq));
+        MXM_BY_STEPS(0, grid);
+        SOMI_LAUNCH_CHECK("mixed_attention_mfma");
+        return 0;
+    }
+    const dim3 grid(n_tokens, splits);
+    MXM_BY_STEPS(1, grid);
+    SOMI_LAUNCH_CHECK("mixed_attention_mfma (statistics)");
+    MXM_BY_STEPS(2, grid);
+    SOMI_LAUNCH_CHECK("mixed_attention_mfma (shares)");
+    const int64_t count = (int64_t)n_tokens * heads * vdim;
+    hipLaunchKernelGGL(mixed_attention_join_kernel, dim3((unsigned)ceil_div64(count, 256)), dim3(256), 0, stream, part, splits,
+                       heads, vdim, positions, v_freq, v_pairing, (bf16*)out, count);
+    SOMI_LAUNCH_CHECK("mixed_attention_join");
+#undef MXM_BY_STEPS
 #undef MXM_BY_ACC
 #undef MXM_LAUNCH
-    SOMI_LAUNCH_CHECK("mixed_attention_mfma");
     return 0;
 }

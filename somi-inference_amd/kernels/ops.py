@@ -1582,13 +1582,19 @@ def mixed_attention_mfma_supported(q: torch.Tensor, k_cache: torch.Tensor, v_cac
                                                               v_cache.shape[2], k_cache.shape[2]))
 
 
+MIXED_SPLIT_KEYS = 64          # a key split of the matrix-core kernel holds at least this many keys
+MIXED_MAX_SPLITS = 64
+
+
 def mixed_attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                          token_entry: torch.Tensor, positions: torch.Tensor, heads: int, window: int, scale: float,
                          softcap: float, denominator_extra: float, talk: torch.Tensor | None,
-                         value_freq: torch.Tensor | None, value_pairing: str = "half", portions: bool = False) -> torch.Tensor:
+                         value_freq: torch.Tensor | None, value_pairing: str = "half", portions: bool = False,
+                         max_context: int = 0) -> torch.Tensor:
     """:func:`mixed_attention_plain` on the matrix cores (bfloat16).  ``portions``: the step holds prompt portions, and
     consecutive tokens share a workgroup (as many as fill 16 query slots a key/value head), so that it reads a tile of
-    keys once for all of them; otherwise a workgroup serves one token."""
+    keys once for all of them; otherwise a workgroup serves one token, and where the step's tokens are few a token's
+    keys are dealt out to several workgroups (``max_context``: the longest context of the step, known to the host)."""
     _need(q, "queries", torch.bfloat16)
     n = q.shape[0]
     _need(k_cache, "key pages", torch.bfloat16)
@@ -1606,12 +1612,21 @@ def mixed_attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
         _need(talk, "head mix", torch.float32, (heads, heads))
     if value_freq is not None:
         _need(value_freq, "value rotation frequencies", torch.float32, (vdim // 2,))
+    splits = 1
+    if not portions and n > 0:
+        seen = int(max_context) if window <= 0 else min(int(max_context), int(window) + 31)
+        splits = max(1, min(MIXED_MAX_SPLITS, seen // MIXED_SPLIT_KEYS, (2 * compute_units()) // n))
     out = torch.empty((n, heads * vdim), dtype=torch.bfloat16, device=q.device)
+    stats = part = None
+    if splits > 1:
+        stats = torch.empty((n * splits * heads * 2,), dtype=torch.float32, device=q.device)
+        part = torch.empty((n * splits * heads * vdim,), dtype=torch.float32, device=q.device)
     _check(library().somi_mixed_attention_mfma(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
                                                _ptr(token_entry), _ptr(positions), n, int(heads), kv_heads, dim, vdim, page,
                                                int(window), ctypes.c_float(scale), ctypes.c_float(softcap),
                                                ctypes.c_float(denominator_extra), _ptr(talk), _ptr(value_freq),
-                                               pairing_code(value_pairing), 1 if portions else 0, _ptr(out), _stream()))
+                                               pairing_code(value_pairing), 1 if portions else 0, splits, _ptr(stats),
+                                               _ptr(part), _ptr(out), _stream()))
     return out
 
 

@@ -151,7 +151,7 @@ class MixedHeadsAttention(Mixer):
                 self.pairing, self.value_freq, (self.value_rotation or {}).get("pairing", "half"), self.num_heads,
                 self.num_kv_heads, self.dim, self.value_dim, None if self.shares_cache else keys,
                 None if self.shares_cache else values, self.runtime.dtype)
-        with stage("attention"):
+        with stage("mixed attention"):
             attended = self.attend(q, keys, values, step, view)
         return self.out.deferred(attended)
 
@@ -163,7 +163,8 @@ class MixedHeadsAttention(Mixer):
             return ops.mixed_attention_mfma(q, keys, values, view.block_table, step.token_entry, step.positions,
                                             self.num_heads, self.window or 0, self.scale, self.softcap,
                                             1.0 if self.sink_one else 0.0, self.talk, self.value_freq, pairing,
-                                            portions=step.max_entry_len >= self.PORTION_TOKENS)
+                                            portions=step.max_entry_len >= self.PORTION_TOKENS,
+                                            max_context=step.max_context)
         return ops.mixed_attention_plain(q, keys, values, view.block_table, step.token_entry, step.positions,
                                          self.num_heads, self.window or 0, self.scale, self.softcap,
                                          1.0 if self.sink_one else 0.0, self.talk, self.value_freq,

@@ -168,3 +168,27 @@ def test_metitar_option_runs_both_models_and_leaves_the_default_alone():
         assert "attention" in line[model]["stages"]["prefill_512"] and "recurrence" in line[model]["stages"]["prefill_512"]
     assert "experts gate_up" in line["metitar"]["stages"]["prefill_512"] and line["value"] == line["metitar"]["decode_b8"]["tok_s"]
     assert line["prefill_kernels"]["metitar_attention"]["ms"] > 0 and line["decode_kernels"]["metitar_recurrence"]["ms"] > 0
+
+
+def test_gizilorn_option_runs_the_models_and_leaves_the_default_alone():
+    """``--gizilorn`` runs a Gizilorn model beside the closest Metitar and Qwen2.5-style models and prints one JSON line;
+    the sizes' config.json dicts are what the registry takes."""
+    import bench
+    from somi_inference_amd.config import config_from_dict
+    for sizes in bench.GIZILORN_SIZES:
+        arch, config = config_from_dict(bench.gizilorn_config_dict(sizes))
+        assert arch.name == "Gizilorn" and len(config.layers) == bench.GIZILORN_LAYERS and config.streams == 4
+        assert config.layers[1].mixer.kv_from == 0
+        arch, closest = config_from_dict(bench.gizilorn_closest_config_dict(sizes))
+        assert arch.name == "Metitar" and closest.width == config.width
+        arch, closest = config_from_dict(bench.gizilorn_closest_attention_config_dict(sizes))
+        assert arch.name == "Qwen2ForCausalLM" and closest.hidden_size == config.width
+    done = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gizilorn", "1b", "--steps", "16", "--warmup", "2",
+                           "--prefill-tokens", "512", "--context", "1024"], capture_output=True, text=True, timeout=900, cwd=ROOT)
+    assert done.returncode == 0, done.stderr[-3000:]
+    line = json.loads([row for row in done.stdout.splitlines() if row.startswith("{")][-1])
+    for model in ("gizilorn", "closest", "closest_attention"):
+        assert line[model]["decode_b8"]["tok_s"] > 0 and line[model]["prefill"]["512"]["tok_s"] > 0
+    assert "mixed attention" in line["gizilorn"]["stages"]["prefill_512"] and line["value"] == line["gizilorn"]["decode_b8"]["tok_s"]
+    assert line["prefill_kernels"]["gizilorn_attention"]["ms"] > 0 and line["decode_kernels"]["gizilorn_latent_attention"]["ms"] > 0
+    assert line["prefill_kernels"]["gizilorn_streams"]["gbs"] > 0

@@ -411,5 +411,8 @@ def test_matrix_core_and_plain_attention_agree(portions, heads, kv, dim, vdim, w
     freq = (1.0 / (50.0 ** (torch.arange(0, vdim, 2, dtype=torch.float64) / vdim))).float().to(DEV)
     args = (q, keys, values, table, entry, position, heads, window or 0, dim ** -0.5, cap or 0.0, 1.0, talk, freq, "half")
     want = ops.mixed_attention_plain(*args)
-    got = ops.mixed_attention_mfma(*args, portions=portions)
+    got = ops.mixed_attention_mfma(*args, portions=portions, max_context=91)
     check(got, want, torch.bfloat16)
+    if not portions:
+        # a token's keys dealt out to several workgroups (as a step of few tokens with long contexts has them)
+        check(ops.mixed_attention_mfma(*args, portions=False, max_context=4096), want, torch.bfloat16)
