@@ -25,11 +25,12 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 mxm_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float mxm_f32x4;
 
+#define MXM_PAGES 2048         // page ids of a run's keys that are kept in LDS (the walk reads the table itself beyond them)
 #define MXM_WROW 40            // bfloat16 a row of 32 weights takes in LDS (rows stay 16-byte aligned)
 
 // cap * tanh(s / cap) with tanh(x) = 1 - 2 / (1 + exp(2 x)): float32, a handful of instructions
 __device__ __forceinline__ float mxm_cap(float s, float cap, float inv_cap) {
-    return cap > 0.f ? cap * (1.0f - 2.0f / (1.0f + __expf(2.0f * s * inv_cap))) : s;
+    return cap > 0.f ? cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * s * inv_cap))) : s;
 }
 
 // mode 0: a workgroup walks all keys of its tokens and writes their outputs.  Modes 1 and 2 split a token's keys over
@@ -58,6 +59,7 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
     bf16* w_lo = w_hi + (size_t)kv * 16 * MXM_WROW;
     float* ml = reinterpret_cast<float*>(w_lo + (size_t)kv * 16 * MXM_WROW);       // [kv][16][2]
     float* o_s = reinterpret_cast<float*>(mxm_lds);                                // [kv][16][vdim], over all of the above
+    __shared__ int pages_s[MXM_PAGES];         // the run's pages from its first key's page on: one lookup a run, not one a load
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, col = lane & 15, quad = lane >> 4;
     const int group = heads / kv, dts = vdim >> 4;
@@ -66,6 +68,10 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
     const int split = blockIdx.y, splits = gridDim.y;
     const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
     const int my_u = col / rp, my_r = col % rp;          // the token and head-in-group of the slot this lane serves
+    // pages of a power of two of tokens (the usual case) are found by a shift, others by a division
+    const int page_shift = (page_size & (page_size - 1)) == 0 ? __ffs(page_size) - 1 : -1;
+    auto page_index = [&](int key) { return page_shift >= 0 ? key >> page_shift : key / page_size; };
+    auto page_offset = [&](int key) { return page_shift >= 0 ? key & (page_size - 1) : key % page_size; };
 
     for (int r0 = 0; r0 < count;) {
         const int entry = token_entry[t0 + r0];
@@ -82,6 +88,12 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
         const int my_pos = live ? positions[t0 + my_u] : -1;
         const int my_first = window > 0 ? max(0, my_pos - window + 1) : 0;
 
+        const int page0 = page_index(kb0);
+        for (int i = tid; i < MXM_PAGES && (int64_t)(page0 + i) * page_size <= p_last; i += 256) pages_s[i] = table[page0 + i];
+        auto page_of = [&](int key) -> int64_t {
+            const int at = page_index(key) - page0;
+            return at < MXM_PAGES ? pages_s[at] : table[page0 + at];
+        };
         // ---- into LDS (the end of a run writes over all of it): the mix in two bfloat16 halves, zeros where weights
         //      of dead slots and padded heads would stand, and the queries of the run's tokens, slot by slot
         for (int i = tid; i < hp * trow; i += 256) {
@@ -107,21 +119,26 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
         __syncthreads();
 
         // scores of 16 keys from kb on against the 16 slots of key/value head c: the lane's 4 keys of its slot
-        auto scores = [&](int c, int kb, float (&s4)[4]) {
+        // the K fragments of 16 keys from kb on of key/value head c (the lane's key row), as they are stored: nothing
+        // touches them until the products that read them, so two tiles' loads are under way at once
+        auto load_keys = [&](int c, int kb, mxm_bf16x8 (&kf)[STEPS]) {
             const int key_row = min(kb + col, p_last);
-            const int64_t page = table[key_row / page_size];
-            const bf16* krow = k_cache + ((page * kv + c) * page_size + key_row % page_size) * dim;
-            const bf16* q_lane = q_s + ((size_t)c * 16 + col) * QROW + quad * 8;
-            mxm_f32x4 sc = mxm_f32x4{0.f, 0.f, 0.f, 0.f};
+            const int64_t page = page_of(key_row);
+            const bf16* krow = k_cache + ((page * kv + c) * page_size + page_offset(key_row)) * dim;
 #pragma unroll
             for (int s = 0; s < STEPS; ++s) {
                 const int ch = s * 32 + quad * 8;
-                mxm_bf16x8 kf;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) kf[e] = (__bf16)0.f;
-                if (ch < dim) kf = *reinterpret_cast<const mxm_bf16x8*>(krow + ch);
-                sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, *reinterpret_cast<const mxm_bf16x8*>(q_lane + s * 32), sc, 0, 0, 0);
+                for (int e = 0; e < 8; ++e) kf[s][e] = (__bf16)0.f;
+                if (ch < dim) kf[s] = *reinterpret_cast<const mxm_bf16x8*>(krow + ch);
             }
+        };
+        auto scores = [&](int c, int kb, const mxm_bf16x8 (&kf)[STEPS], float (&s4)[4]) {
+            const bf16* q_lane = q_s + ((size_t)c * 16 + col) * QROW + quad * 8;
+            mxm_f32x4 sc = mxm_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+                sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[s], *reinterpret_cast<const mxm_bf16x8*>(q_lane + s * 32), sc, 0, 0, 0);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int key = kb + quad * 4 + i;
@@ -133,15 +150,21 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
         for (int c = w; c < kv; c += 4) {
             float m = -INFINITY, l = 0.f;
             if (mode != 2) {
-                for (int kb = kb0; kb <= k_hi; kb += 16) {
-                    float s4[4];
-                    scores(c, kb, s4);
-                    const float mx = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
-                    const float m_new = fmaxf(m, mx);
-                    if (m_new > -INFINITY) {
-                        l = l * __expf(m - m_new) + ((__expf(s4[0] - m_new) + __expf(s4[1] - m_new)) +
-                                                    (__expf(s4[2] - m_new) + __expf(s4[3] - m_new)));
-                        m = m_new;
+                for (int kb = kb0; kb <= k_hi; kb += 32) {
+                    mxm_bf16x8 kf[2][STEPS];
+                    load_keys(c, kb, kf[0]);
+                    load_keys(c, kb + 16, kf[1]);
+#pragma unroll
+                    for (int x = 0; x < 2; ++x) {
+                        float s4[4];
+                        scores(c, kb + 16 * x, kf[x], s4);
+                        const float mx = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
+                        const float m_new = fmaxf(m, mx);
+                        if (m_new > -INFINITY) {
+                            l = l * __expf(m - m_new) + ((__expf(s4[0] - m_new) + __expf(s4[1] - m_new)) +
+                                                        (__expf(s4[2] - m_new) + __expf(s4[3] - m_new)));
+                            m = m_new;
+                        }
                     }
                 }
             } else if (live && quad == 0) {
@@ -191,11 +214,14 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
             // the weights p = exp(s - m) / l, by (token, key) and head, in two bfloat16 halves
             for (int c = w; c < kv; c += 4) {
                 const float m = ml[(c * 16 + col) * 2], inv_l = live ? 1.0f / ml[(c * 16 + col) * 2 + 1] : 0.f;
+                mxm_bf16x8 kf[2][STEPS];
+                load_keys(c, kb, kf[0]);
+                load_keys(c, kb + 16, kf[1]);
                 // every lane takes part in the scores (its key row is one of the tile's 16, whatever its slot is)
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
                     float s4[4];
-                    scores(c, kb + half * 16, s4);
+                    scores(c, kb + half * 16, kf[half], s4);
                     if (live) {
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
@@ -243,8 +269,8 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
             __syncthreads();
             // the lane's 8 keys lie in one page (pages hold a multiple of 8 tokens, the walk is aligned to 32)
             const int key8 = min(kb + quad * 8, p_last & ~7);
-            const int64_t page = table[key8 / page_size];
-            const int off = key8 % page_size;
+            const int64_t page = page_of(key8);
+            const int off = page_offset(key8);
 #pragma unroll
             for (int a = 0; a < ACC; ++a) {
                 const int pair = w + 4 * a;
@@ -352,14 +378,14 @@ extern "C" int somi_mixed_attention_mfma_supported(int heads, int kv, int dim, i
 // As somi_mixed_attention_plain, bfloat16 only.  portions != 0: the step holds prompt portions, and as many consecutive
 // tokens share a workgroup as their heads fill 16 query slots a key/value head; otherwise a workgroup serves one token,
 // and with splits > 1 a token's keys are dealt out to that many workgroups (three launches: the splits' statistics,
-// their shares of the output, the join), for which `stats` holds n_tokens * splits * heads * 2 floats and `part`
+// their shares of the output, the join; group_tokens must be 0 then), for which `stats` holds n_tokens * splits * heads * 2 floats and `part`
 // n_tokens * splits * heads * vdim.
 extern "C" int somi_mixed_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int* block_table,
                                          int max_blocks, const int* token_entry, const int* positions, int n_tokens,
                                          int heads, int kv, int dim, int vdim, int page_size, int window, float scale,
                                          float cap, float extra, const float* talk, const float* v_freq, int v_pairing,
                                          int portions, int splits, float* stats, float* part, void* out,
-                                         hipStream_t stream) {
+                                         int group_tokens, hipStream_t stream) {
     SOMI_REQUIRE(n_tokens >= 0 && max_blocks > 0 && window >= 0 && splits >= 1 && splits <= 65535, "mixed_attention_mfma: bad sizes");
     SOMI_REQUIRE(somi_mixed_attention_mfma_supported(heads, kv, dim, vdim, page_size),
                  "mixed_attention_mfma: %d heads over %d of %d + %d channels in pages of %d are not what the kernel is built for",
@@ -372,7 +398,10 @@ extern "C" int somi_mixed_attention_mfma(const void* q, const void* k_cache, con
     const int group = heads / kv;
     int rp = 1;
     while (rp < group) rp <<= 1;
-    const int tq = portions ? 16 / rp : 1;
+    // tokens a workgroup: at most what fills the 16 slots; fewer tokens make more workgroups, whose waits for memory
+    // overlap (group_tokens: the caller's choice, 0 = the default)
+    int tq = portions ? 16 / rp : 1;
+    if (portions && group_tokens > 0 && group_tokens < tq) tq = group_tokens;
     const int steps = mxm_steps(dim), accs = mxm_acc(kv, vdim);
     const size_t lds = mxm_lds_bytes(steps, heads, kv, vdim, tq);
 #define MXM_LAUNCH(STEPS, ACC, MODE, GRID)                                                                              \

@@ -1590,7 +1590,7 @@ def mixed_attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
                          token_entry: torch.Tensor, positions: torch.Tensor, heads: int, window: int, scale: float,
                          softcap: float, denominator_extra: float, talk: torch.Tensor | None,
                          value_freq: torch.Tensor | None, value_pairing: str = "half", portions: bool = False,
-                         max_context: int = 0) -> torch.Tensor:
+                         max_context: int = 0, group_tokens: int = 0) -> torch.Tensor:
     """:func:`mixed_attention_plain` on the matrix cores (bfloat16).  ``portions``: the step holds prompt portions, and
     consecutive tokens share a workgroup (as many as fill 16 query slots a key/value head), so that it reads a tile of
     keys once for all of them; otherwise a workgroup serves one token, and where the step's tokens are few a token's
@@ -1626,7 +1626,7 @@ def mixed_attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
                                                int(window), ctypes.c_float(scale), ctypes.c_float(softcap),
                                                ctypes.c_float(denominator_extra), _ptr(talk), _ptr(value_freq),
                                                pairing_code(value_pairing), 1 if portions else 0, splits, _ptr(stats),
-                                               _ptr(part), _ptr(out), _stream()))
+                                               _ptr(part), _ptr(out), int(group_tokens), _stream()))
     return out
 
 
