@@ -186,17 +186,24 @@ template <typename TO>
 __global__ void __launch_bounds__(256)
 xielu_kernel(const float* __restrict__ z, const float* __restrict__ pq, TO* __restrict__ out, int64_t count) {
     const float ap = somi_softplus(pq[0]), an = 0.5f + somi_softplus(pq[1]);
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t)gridDim.x * 256) {
-        const float v = z[i];
-        const float r = v > 0.f ? fmaf(ap * v, v, 0.5f * v) : fmaf(an, expm1f(v) - v, 0.5f * v);
-        out[i] = from_float<TO>(r);
+    auto unit = [&](float v) { return v > 0.f ? fmaf(ap * v, v, 0.5f * v) : fmaf(an, expm1f(v) - v, 0.5f * v); };
+    // four values a thread and round (16 bytes in), then what is left one by one
+    const int64_t quads = count >> 2;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < quads; i += (int64_t)gridDim.x * 256) {
+        const float4 v = reinterpret_cast<const float4*>(z)[i];
+        TO r[4] = {from_float<TO>(unit(v.x)), from_float<TO>(unit(v.y)), from_float<TO>(unit(v.z)), from_float<TO>(unit(v.w))};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[i * 4 + e] = r[e];
     }
+    for (int64_t i = quads * 4 + (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t)gridDim.x * 256)
+        out[i] = from_float<TO>(unit(z[i]));
 }
 
 extern "C" int somi_xielu(const float* z, const float* pq, void* out, int out_dtype, int64_t count, hipStream_t stream) {
     SOMI_REQUIRE(count >= 0, "xielu: bad sizes");
+    SOMI_REQUIRE(((uintptr_t)z & 15) == 0, "xielu: rows must start at a multiple of 16 bytes");
     if (count == 0) return 0;
-    const int grid = (int)(ceil_div64(count, 256) < 65536 ? ceil_div64(count, 256) : 65536);
+    const int grid = (int)(ceil_div64(count, 1024) < 65536 ? ceil_div64(count, 1024) : 65536);
     if (out_dtype == SOMI_F32)
         hipLaunchKernelGGL(xielu_kernel<float>, dim3(grid), dim3(256), 0, stream, z, pq, (float*)out, count);
     else if (out_dtype == SOMI_BF16)

@@ -16,7 +16,8 @@
 #define HC_MAX_STREAMS 8
 #define HC_NT 256
 
-template <typename TY, typename TO>
+// VEC: columns a thread takes at a time (4 where the width is a multiple of 4: 16-byte accesses of the streams).
+template <typename TY, typename TO, int VEC>
 __global__ void __launch_bounds__(HC_NT)
 hc_step_kernel(float* __restrict__ lanes, int S, int64_t n, int width, const float* __restrict__ mix,
                const float* __restrict__ out_w, const TY* __restrict__ y, const float* __restrict__ in_w, int read,
@@ -37,51 +38,73 @@ hc_step_kernel(float* __restrict__ lanes, int S, int64_t n, int width, const flo
     const int64_t plane = n * (int64_t)width;
     float* base = lanes + row * width;
     float ss = 0.f;
-    for (int c = tid; c < width; c += HC_NT) {
-        float x[HC_MAX_STREAMS];
+    for (int c = tid * VEC; c < width; c += HC_NT * VEC) {
+        float x[HC_MAX_STREAMS][VEC];
 #pragma unroll
         for (int s = 0; s < HC_MAX_STREAMS; ++s)
-            if (s < S) x[s] = base[s * plane + c];
+            if (s < S) {
+                if (VEC == 4) {
+                    const float4 v = *reinterpret_cast<const float4*>(base + s * plane + c);
+                    x[s][0] = v.x; x[s][1] = v.y; x[s][2 % VEC] = v.z; x[s][3 % VEC] = v.w;
+                } else {
+                    x[s][0] = base[s * plane + c];
+                }
+            }
         if (y != nullptr) {
-            const float yv = to_float(y[row * width + c]);
-            float fresh[HC_MAX_STREAMS];
+            float yv[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) yv[e] = to_float(y[row * width + c + e]);
+            float fresh[HC_MAX_STREAMS][VEC];
 #pragma unroll
             for (int t = 0; t < HC_MAX_STREAMS; ++t)
                 if (t < S) {
-                    float v = 0.f;
 #pragma unroll
-                    for (int s = 0; s < HC_MAX_STREAMS; ++s)
-                        if (s < S) v = fmaf(m_s[s * S + t], x[s], v);
-                    fresh[t] = fmaf(b_s[t], yv, v);
+                    for (int e = 0; e < VEC; ++e) {
+                        float v = 0.f;
+#pragma unroll
+                        for (int s = 0; s < HC_MAX_STREAMS; ++s)
+                            if (s < S) v = fmaf(m_s[s * S + t], x[s][e], v);
+                        fresh[t][e] = fmaf(b_s[t], yv[e], v);
+                    }
                 }
 #pragma unroll
             for (int t = 0; t < HC_MAX_STREAMS; ++t)
                 if (t < S) {
-                    x[t] = fresh[t];
-                    base[t * plane + c] = fresh[t];
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) x[t][e] = fresh[t][e];
+                    if (VEC == 4)
+                        *reinterpret_cast<float4*>(base + t * plane + c) = make_float4(fresh[t][0], fresh[t][1 % VEC], fresh[t][2 % VEC], fresh[t][3 % VEC]);
+                    else
+                        base[t * plane + c] = fresh[t][0];
                 }
         }
         if (read) {
-            float u = 0.f;
 #pragma unroll
-            for (int s = 0; s < HC_MAX_STREAMS; ++s)
-                if (s < S) u = fmaf(a_s[s], x[s], u);
-            ss = fmaf(u, u, ss);
-            if (norm_w == nullptr)
-                for (int k = 0; k < copies; ++k) out[k * plane + row * width + c] = from_float<TO>(u);
+            for (int e = 0; e < VEC; ++e) {
+                float u = 0.f;
+#pragma unroll
+                for (int s = 0; s < HC_MAX_STREAMS; ++s)
+                    if (s < S) u = fmaf(a_s[s], x[s][e], u);
+                ss = fmaf(u, u, ss);
+                if (norm_w == nullptr)
+                    for (int k = 0; k < copies; ++k) out[k * plane + row * width + c + e] = from_float<TO>(u);
+            }
         }
     }
     if (!read || norm_w == nullptr) return;
     ss = block_sum<HC_NT>(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)width + eps);
     // the sums once more, from the values this thread itself has just written (or only read)
-    for (int c = tid; c < width; c += HC_NT) {
-        float u = 0.f;
+    for (int c = tid * VEC; c < width; c += HC_NT * VEC) {
 #pragma unroll
-        for (int s = 0; s < HC_MAX_STREAMS; ++s)
-            if (s < S) u = fmaf(a_s[s], base[s * plane + c], u);
-        const TO v = from_float<TO>(u * inv * norm_w[c]);
-        for (int k = 0; k < copies; ++k) out[k * plane + row * width + c] = v;
+        for (int e = 0; e < VEC; ++e) {
+            float u = 0.f;
+#pragma unroll
+            for (int s = 0; s < HC_MAX_STREAMS; ++s)
+                if (s < S) u = fmaf(a_s[s], base[s * plane + c + e], u);
+            const TO v = from_float<TO>(u * inv * norm_w[c + e]);
+            for (int k = 0; k < copies; ++k) out[k * plane + row * width + c + e] = v;
+        }
     }
 }
 
@@ -89,8 +112,12 @@ template <typename TY, typename TO>
 static void hc_launch(float* lanes, int S, int64_t n, int width, const float* mix, const float* out_w, const void* y,
                       const float* in_w, int read, const float* norm_w, float eps, void* out, int copies,
                       hipStream_t stream) {
-    hipLaunchKernelGGL((hc_step_kernel<TY, TO>), dim3((unsigned)n), dim3(HC_NT), 0, stream, lanes, S, n, width, mix, out_w,
-                       (const TY*)y, in_w, read, norm_w, eps, (TO*)out, copies);
+    if (width % 4 == 0 && ((uintptr_t)lanes & 15) == 0)
+        hipLaunchKernelGGL((hc_step_kernel<TY, TO, 4>), dim3((unsigned)n), dim3(HC_NT), 0, stream, lanes, S, n, width, mix,
+                           out_w, (const TY*)y, in_w, read, norm_w, eps, (TO*)out, copies);
+    else
+        hipLaunchKernelGGL((hc_step_kernel<TY, TO, 1>), dim3((unsigned)n), dim3(HC_NT), 0, stream, lanes, S, n, width, mix,
+                           out_w, (const TY*)y, in_w, read, norm_w, eps, (TO*)out, copies);
 }
 
 // y: [n, width] of y_dtype or null (then mix and out_w are not read).  read != 0: out gets the (normed) sum, in

@@ -35,7 +35,7 @@ def check(got, want, dtype, loose=1.0):
 
 # ------------------------------------------------------------------------------------------ the streams
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("streams,width,rows", [(1, 8, 3), (2, 100, 17), (3, 96, 5), (4, 1000, 9), (8, 260, 2)])
+@pytest.mark.parametrize("streams,width,rows", [(1, 8, 3), (2, 100, 17), (3, 96, 5), (4, 1000, 9), (8, 260, 2), (3, 7, 4), (2, 1030, 3)])
 def test_streams_read_write_and_both_in_one_launch(dtype, streams, width, rows):
     gen = torch.Generator().manual_seed(streams * width)
     lanes = torch.randn(streams, rows, width, generator=gen) * 3
