@@ -266,9 +266,16 @@ extern "C" int somi_mixed_attention_plain(const void* q, int dtype, const void* 
     const size_t floats = (size_t)heads * dim + (size_t)heads * heads + 2 * heads + 2 * (size_t)heads * MXA_TILE +
                           (((size_t)heads * vdim + 1) & ~(size_t)1);
     const size_t smem = floats * sizeof(float) + MXA_TILE * sizeof(int64_t);
-    SOMI_REQUIRE(smem <= 64 * 1024, "mixed_attention: %d heads of %d + %d channels need %zu bytes of LDS, more than 64 KiB",
+    SOMI_REQUIRE(smem <= 160 * 1024, "mixed_attention: %d heads of %d + %d channels need %zu bytes of LDS, more than 160 KiB",
                  heads, dim, vdim, smem);
     const dim3 grid(n_tokens);
+    if (smem > 48 * 1024) {
+        // more LDS than a workgroup gets unasked
+        const void* kernel = dtype == SOMI_F32 ? (const void*)mixed_attention_plain_kernel<float>
+                                               : (const void*)mixed_attention_plain_kernel<bf16>;
+        hipError_t err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (err != hipSuccess) return somi_fail("mixed_attention: %s", hipGetErrorString(err));
+    }
     if (dtype == SOMI_F32)
         hipLaunchKernelGGL(mixed_attention_plain_kernel<float>, grid, dim3(MXA_NT), smem, stream, (const float*)q,
                            (const float*)k_cache, (const float*)v_cache, block_table, max_blocks, token_entry, positions,

@@ -416,3 +416,16 @@ def test_matrix_core_and_plain_attention_agree(portions, heads, kv, dim, vdim, w
     if not portions:
         # a token's keys dealt out to several workgroups (as a step of few tokens with long contexts has them)
         check(ops.mixed_attention_mfma(*args, portions=False, max_context=4096), want, torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_many_wide_heads_in_the_plain_kernel(dtype):
+    """64 heads of 64 + 64 channels: more LDS than a workgroup gets unasked, and (in bfloat16) more query heads a
+    key/value head than the matrix-core kernel has slots."""
+    part, m = mixed_part(64, 2, 64, 64, 20, 10.0, 32)
+    w = mixed_weights(part, 5)
+    load_part(part, w, dtype, DEV)
+    x = rounded(torch.randn(45, 48, generator=torch.Generator().manual_seed(3)), dtype)
+    want = plain.attention(x, w, "m.", m)
+    engine = PartEngine([part], dtype, DEV, 16, num_blocks=8)
+    check(engine.run_cut("a", x, [30, 1, 14])[0], want, dtype)
