@@ -1,12 +1,12 @@
 // Attention with mixed heads on the matrix cores (bfloat16): see mixed_attention.hip for what is computed.
 //
-// A workgroup (four wavefronts) serves `tq` consecutive tokens of the step and ALL their heads, because the mix needs
+// A workgroup (eight wavefronts) serves `tq` consecutive tokens of the step and ALL their heads, because the mix needs
 // every head's weights of a (token, key) pair in one place.  For each key/value head c there is one tile of 16 query
 // slots: slot = token * rp + r holds head c * group + r of that token (rp: the power of two >= group; slots with r >=
 // group, or of tokens of another request, are dead).  Tokens of one request stand side by side with rising positions;
 // where the workgroup's tokens belong to several requests it takes them run by run.
 //
-//   first walk   wavefront w takes the key/value heads w, w + 4, ...; 16 keys at a time, S^T = K Q^T by `16x16x32`
+//   first walk   a wavefront takes a (key/value head, parity of the 16-key tile) at a time; 16 keys at a time, S^T = K Q^T by `16x16x32`
 //                products (K fragments straight from the pages, Q fragments from LDS); a lane holds 4 keys of one slot
 //                and keeps a running maximum and sum of its own, joined over the lanes at the end: (m, l) of every slot
 //   second walk  32 keys at a time: the same scores again, p = exp(s - m) / l in float32, which goes to LDS by (token,
@@ -26,7 +26,16 @@ typedef __attribute__((ext_vector_type(8))) __bf16 mxm_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float mxm_f32x4;
 
 #define MXM_PAGES 2048         // page ids of a run's keys that are kept in LDS (the walk reads the table itself beyond them)
+#define MXM_NW 8               // wavefronts of a workgroup
+#define MXM_NT (64 * MXM_NW)
 #define MXM_WROW 40            // bfloat16 a row of 32 weights takes in LDS (rows stay 16-byte aligned)
+
+// A barrier for data that went through LDS: waits for this wavefront's LDS traffic only, so that loads from memory
+// that were asked for ahead of their use stay in flight across it (the language's barrier waits for those as well).
+__device__ __forceinline__ void mxm_lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+}
 
 // cap * tanh(s / cap) with tanh(x) = 1 - 2 / (1 + exp(2 x)): float32, a handful of instructions
 __device__ __forceinline__ float mxm_cap(float s, float cap, float inv_cap) {
@@ -39,7 +48,7 @@ __device__ __forceinline__ float mxm_cap(float s, float cap, float inv_cap) {
 // weights of its keys against the joined maximum and sum, and leaves its unnormed share of the output, which is simply a
 // term of the sum over the splits, in `part` [tokens, splits, heads * vdim] (not yet turned back).
 template <int STEPS, int ACC>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(MXM_NT)
 mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
                             const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_entry,
                             const int* __restrict__ positions, int n_tokens, int heads, int kv, int dim, int vdim,
@@ -58,6 +67,7 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
     bf16* w_hi = p_lo + (size_t)tq * 32 * trow;                                    // [kv][16][WROW]
     bf16* w_lo = w_hi + (size_t)kv * 16 * MXM_WROW;
     float* ml = reinterpret_cast<float*>(w_lo + (size_t)kv * 16 * MXM_WROW);       // [kv][16][2]
+    float* ml_half = ml + (size_t)kv * 32;                                         // [kv][2 (tile parity)][16][2]
     float* o_s = reinterpret_cast<float*>(mxm_lds);                                // [kv][16][vdim], over all of the above
     __shared__ int pages_s[MXM_PAGES];         // the run's pages from its first key's page on: one lookup a run, not one a load
 
@@ -89,14 +99,14 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
         const int my_first = window > 0 ? max(0, my_pos - window + 1) : 0;
 
         const int page0 = page_index(kb0);
-        for (int i = tid; i < MXM_PAGES && (int64_t)(page0 + i) * page_size <= p_last; i += 256) pages_s[i] = table[page0 + i];
+        for (int i = tid; i < MXM_PAGES && (int64_t)(page0 + i) * page_size <= p_last; i += MXM_NT) pages_s[i] = table[page0 + i];
         auto page_of = [&](int key) -> int64_t {
             const int at = page_index(key) - page0;
             return at < MXM_PAGES ? pages_s[at] : table[page0 + at];
         };
         // ---- into LDS (the end of a run writes over all of it): the mix in two bfloat16 halves, zeros where weights
         //      of dead slots and padded heads would stand, and the queries of the run's tokens, slot by slot
-        for (int i = tid; i < hp * trow; i += 256) {
+        for (int i = tid; i < hp * trow; i += MXM_NT) {
             const int h = i / trow, g = i % trow;
             float t = 0.f;
             if (h < heads && g < heads) t = talk != nullptr ? talk[h * heads + g] : (h == g ? 1.f : 0.f);
@@ -104,9 +114,9 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
             t_hi[i] = hi;
             t_lo[i] = (bf16)(t - (float)hi);
         }
-        for (int i = tid; i < tq * 32 * trow; i += 256) p_hi[i] = p_lo[i] = (bf16)0.f;
-        for (int i = tid; i < kv * 16 * MXM_WROW; i += 256) w_hi[i] = w_lo[i] = (bf16)0.f;
-        for (int i = tid; i < kv * 16 * STEPS * 4; i += 256) {
+        for (int i = tid; i < tq * 32 * trow; i += MXM_NT) p_hi[i] = p_lo[i] = (bf16)0.f;
+        for (int i = tid; i < kv * 16 * MXM_WROW; i += MXM_NT) w_hi[i] = w_lo[i] = (bf16)0.f;
+        for (int i = tid; i < kv * 16 * STEPS * 4; i += MXM_NT) {
             const int ch = (i % (STEPS * 4)) * 8, slot = (i / (STEPS * 4)) % 16, c = i / (STEPS * 4 * 16);
             const int u = slot / rp, r = slot % rp;
             mxm_bf16x8 v;
@@ -146,18 +156,21 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
             }
         };
 
-        // ---- first walk: every slot's maximum and sum (mode 2: joined from what the splits left)
-        for (int c = w; c < kv; c += 4) {
-            float m = -INFINITY, l = 0.f;
-            if (mode != 2) {
-                for (int kb = kb0; kb <= k_hi; kb += 32) {
-                    mxm_bf16x8 kf[2][STEPS];
-                    load_keys(c, kb, kf[0]);
-                    load_keys(c, kb + 16, kf[1]);
+        // ---- first walk: every slot's maximum and sum.  A unit of work is (key/value head, parity of the 16-key tile);
+        //      the two parities' results are joined afterwards (mode 2: the splits' results are joined instead)
+        if (mode != 2) {
+            for (int unit = w; unit < kv * 2; unit += MXM_NW) {
+                const int c = unit >> 1, parity = unit & 1;
+                float m = -INFINITY, l = 0.f;
+                // four tiles of this parity a round: all their fragments are asked for before the first is used
+                for (int kb = kb0 + 16 * parity; kb <= k_hi; kb += 128) {
+                    mxm_bf16x8 kf[4][STEPS];
 #pragma unroll
-                    for (int x = 0; x < 2; ++x) {
+                    for (int x = 0; x < 4; ++x) load_keys(c, kb + 32 * x, kf[x]);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
                         float s4[4];
-                        scores(c, kb + 16 * x, kf[x], s4);
+                        scores(c, kb + 32 * x, kf[x], s4);
                         const float mx = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
                         const float m_new = fmaxf(m, mx);
                         if (m_new > -INFINITY) {
@@ -167,37 +180,49 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
                         }
                     }
                 }
-            } else if (live && quad == 0) {
-                const float* mine = stats + (((int64_t)(t0 + my_u) * splits) * heads + c * group + my_r) * 2;
-                for (int s = 0; s < splits; ++s) {
-                    const float m_s = mine[(int64_t)s * heads * 2], l_s = mine[(int64_t)s * heads * 2 + 1];
-                    const float m_new = fmaxf(m, m_s);
-                    if (m_new > -INFINITY) {
-                        l = l * __expf(m - m_new) + l_s * __expf(m_s - m_new);
-                        m = m_new;
-                    }
+                // the four lanes of a slot
+                float top = fmaxf(m, __shfl_xor(m, 16, 64));
+                top = fmaxf(top, __shfl_xor(top, 32, 64));
+                float sum = top > -INFINITY ? l * __expf(m - top) : 0.f;
+                sum += __shfl_xor(sum, 16, 64);
+                sum += __shfl_xor(sum, 32, 64);
+                if (quad == 0) {
+                    ml_half[(unit * 16 + col) * 2] = top;
+                    ml_half[(unit * 16 + col) * 2 + 1] = sum;
                 }
             }
-            // the four lanes of a slot, then the sink's share
-            float top = fmaxf(m, __shfl_xor(m, 16, 64));
-            top = fmaxf(top, __shfl_xor(top, 32, 64));
-            if (extra > 0.f && mode != 1) top = fmaxf(top, 0.f);
-            float sum = top > -INFINITY ? l * __expf(m - top) : 0.f;
-            sum += __shfl_xor(sum, 16, 64);
-            sum += __shfl_xor(sum, 32, 64);
-            if (extra > 0.f && mode != 1) sum += extra * __expf(-top);
-            if (quad == 0) {
-                if (mode == 1) {
-                    if (live) {
-                        float* mine = stats + ((((int64_t)(t0 + my_u) * splits + split) * heads) + c * group + my_r) * 2;
-                        mine[0] = top;
-                        mine[1] = sum;
-                    }
-                } else {
-                    ml[(c * 16 + col) * 2] = top;
-                    ml[(c * 16 + col) * 2 + 1] = sum;
+            __syncthreads();
+        }
+        // a thread a (key/value head, slot): the parities (or the splits) joined, then the sink's share
+        for (int i = tid; i < kv * 16; i += MXM_NT) {
+            const int c = i >> 4, slot = i & 15, u = slot / rp, r = slot % rp;
+            const bool mine = u >= r0 && u < r1 && r < group;
+            float m = -INFINITY, l = 0.f;
+            auto join = [&](float m_s, float l_s) {
+                const float m_new = fmaxf(m, m_s);
+                if (m_new > -INFINITY) {
+                    l = l * __expf(m - m_new) + l_s * __expf(m_s - m_new);
+                    m = m_new;
                 }
+            };
+            if (mode != 2) {
+                join(ml_half[((c * 2) * 16 + slot) * 2], ml_half[((c * 2) * 16 + slot) * 2 + 1]);
+                join(ml_half[((c * 2 + 1) * 16 + slot) * 2], ml_half[((c * 2 + 1) * 16 + slot) * 2 + 1]);
+            } else if (mine) {
+                const float* from = stats + (((int64_t)(t0 + u) * splits) * heads + c * group + r) * 2;
+                for (int sp = 0; sp < splits; ++sp) join(from[(int64_t)sp * heads * 2], from[(int64_t)sp * heads * 2 + 1]);
             }
+            if (mode == 1) {
+                if (mine) {
+                    float* to = stats + ((((int64_t)(t0 + u) * splits + split) * heads) + c * group + r) * 2;
+                    to[0] = m;
+                    to[1] = l;
+                }
+                continue;
+            }
+            if (extra > 0.f) join(0.f, extra);
+            ml[i * 2] = m;
+            ml[i * 2 + 1] = l;
         }
         if (mode == 1) {
             __syncthreads();
@@ -210,18 +235,40 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
         mxm_f32x4 acc[ACC];
 #pragma unroll
         for (int a = 0; a < ACC; ++a) acc[a] = mxm_f32x4{0.f, 0.f, 0.f, 0.f};
+        // the K fragments of the wavefront's first unit are asked for a chunk ahead, a chunk's V^T fragments at its top:
+        // both are under way while the chunk's weights go through LDS (whose barriers wait for LDS only)
+        mxm_bf16x8 kf_ahead[STEPS];
+        if (w < kv * 2 && kb0 <= k_hi) load_keys(w >> 1, kb0 + (w & 1) * 16, kf_ahead);
         for (int kb = kb0; kb <= k_hi; kb += 32) {
-            // the weights p = exp(s - m) / l, by (token, key) and head, in two bfloat16 halves
-            for (int c = w; c < kv; c += 4) {
-                const float m = ml[(c * 16 + col) * 2], inv_l = live ? 1.0f / ml[(c * 16 + col) * 2 + 1] : 0.f;
-                mxm_bf16x8 kf[2][STEPS];
-                load_keys(c, kb, kf[0]);
-                load_keys(c, kb + 16, kf[1]);
-                // every lane takes part in the scores (its key row is one of the tile's 16, whatever its slot is)
+            mxm_bf16x8 vf[ACC];
+            {
+                // the lane's 8 keys lie in one page (pages hold a multiple of 8 tokens, the walk is aligned to 32)
+                const int key8 = min(kb + quad * 8, p_last & ~7);
+                const int64_t page = page_of(key8);
+                const int off = page_offset(key8);
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {
+                for (int a = 0; a < ACC; ++a) {
+                    const int pair = w + MXM_NW * a;
+                    if (pair < kv * dts)
+                        vf[a] = *reinterpret_cast<const mxm_bf16x8*>(
+                            v_cache + (((page * kv + pair / dts) * vdim + (pair % dts) * 16 + col) * page_size + off));
+                }
+            }
+            // the weights p = exp(s - m) / l, by (token, key) and head, in two bfloat16 halves
+            for (int unit = w; unit < kv * 2; unit += MXM_NW) {
+                const int c = unit >> 1, half = unit & 1;
+                const float m = ml[(c * 16 + col) * 2], inv_l = live ? 1.0f / ml[(c * 16 + col) * 2 + 1] : 0.f;
+                mxm_bf16x8 kf[STEPS];
+                if (unit == w) {
+#pragma unroll
+                    for (int st = 0; st < STEPS; ++st) kf[st] = kf_ahead[st];
+                } else {
+                    load_keys(c, kb + half * 16, kf);
+                }
+                // every lane takes part in the scores (its key row is one of the tile's 16, whatever its slot is)
+                {
                     float s4[4];
-                    scores(c, kb + half * 16, kf[half], s4);
+                    scores(c, kb + half * 16, kf, s4);
                     if (live) {
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
@@ -234,11 +281,12 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
                     }
                 }
             }
-            __syncthreads();
+            if (w < kv * 2 && kb + 32 <= k_hi) load_keys(w >> 1, kb + 32 + (w & 1) * 16, kf_ahead);
+            mxm_lds_barrier();
             // the mix: W^T [(token, key) x head] = P^T [(token, key) x head] T^T, tiles of 16 x 16 over the wavefronts
             {
                 const int n_tiles = tq * 2, h_tiles = (heads + 15) >> 4;
-                for (int tile = w; tile < n_tiles * h_tiles; tile += 4) {
+                for (int tile = w; tile < n_tiles * h_tiles; tile += MXM_NW) {
                     const int nt = tile / h_tiles, ht = tile % h_tiles;
                     mxm_f32x4 mixed = mxm_f32x4{0.f, 0.f, 0.f, 0.f};
                     for (int ks = 0; ks < hp; ks += 32) {
@@ -266,21 +314,14 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
                     }
                 }
             }
-            __syncthreads();
-            // the lane's 8 keys lie in one page (pages hold a multiple of 8 tokens, the walk is aligned to 32)
-            const int key8 = min(kb + quad * 8, p_last & ~7);
-            const int64_t page = page_of(key8);
-            const int off = page_offset(key8);
+            mxm_lds_barrier();
 #pragma unroll
             for (int a = 0; a < ACC; ++a) {
-                const int pair = w + 4 * a;
+                const int pair = w + MXM_NW * a;
                 if (pair < kv * dts) {
-                    const int c = pair / dts, dt = pair % dts;
-                    const mxm_bf16x8 vf = *reinterpret_cast<const mxm_bf16x8*>(
-                        v_cache + (((page * kv + c) * vdim + dt * 16 + col) * page_size + off));
-                    const size_t at = ((size_t)c * 16 + col) * MXM_WROW + quad * 8;
-                    acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, *reinterpret_cast<const mxm_bf16x8*>(w_hi + at), acc[a], 0, 0, 0);
-                    acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, *reinterpret_cast<const mxm_bf16x8*>(w_lo + at), acc[a], 0, 0, 0);
+                    const size_t at = ((size_t)(pair / dts) * 16 + col) * MXM_WROW + quad * 8;
+                    acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[a], *reinterpret_cast<const mxm_bf16x8*>(w_hi + at), acc[a], 0, 0, 0);
+                    acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[a], *reinterpret_cast<const mxm_bf16x8*>(w_lo + at), acc[a], 0, 0, 0);
                 }
             }
         }
@@ -288,7 +329,7 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
         __syncthreads();
 #pragma unroll
         for (int a = 0; a < ACC; ++a) {
-            const int pair = w + 4 * a;
+            const int pair = w + MXM_NW * a;
             if (pair < kv * dts) {
                 const int c = pair / dts, dt = pair % dts;
 #pragma unroll
@@ -296,7 +337,7 @@ mixed_attention_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__
             }
         }
         __syncthreads();
-        for (int i = tid; i < kv * 16 * vdim; i += 256) {
+        for (int i = tid; i < kv * 16 * vdim; i += MXM_NT) {
             const int d = i % vdim, slot = (i / vdim) % 16, c = i / (vdim * 16);
             const int u = slot / rp, r = slot % rp;
             if (u < r0 || u >= r1 || r >= group) continue;
@@ -354,22 +395,22 @@ mixed_attention_join_kernel(const float* __restrict__ part, int splits, int head
 static size_t mxm_lds_bytes(int steps, int heads, int kv, int vdim, int tq) {
     const size_t hp = (size_t)((heads + 31) & ~31), trow = hp + 8;
     const size_t walk = (size_t)kv * 16 * (steps * 32 + 8) * 2 + 2 * hp * trow * 2 + 2 * (size_t)tq * 32 * trow * 2 +
-                        2 * (size_t)kv * 16 * MXM_WROW * 2 + (size_t)kv * 32 * 4;
+                        2 * (size_t)kv * 16 * MXM_WROW * 2 + (size_t)kv * 32 * 4 + (size_t)kv * 64 * 4;
     const size_t end = (size_t)kv * 16 * vdim * 4;
     return walk > end ? walk : end;
 }
 
 static int mxm_steps(int dim) { return dim <= 32 ? 1 : dim <= 64 ? 2 : dim <= 128 ? 4 : 8; }
 static int mxm_acc(int kv, int vdim) {
-    const int need = ceil_div(kv * (vdim / 16), 4);
-    return need <= 2 ? 2 : need <= 4 ? 4 : need <= 8 ? 8 : 16;
+    const int need = ceil_div(kv * (vdim / 16), MXM_NW);
+    return need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : 8;
 }
 
 extern "C" int somi_mixed_attention_mfma_supported(int heads, int kv, int dim, int vdim, int page_size) {
     if (heads <= 0 || kv <= 0 || heads % kv || heads / kv > 16 || dim <= 0 || dim % 8 || dim > 256 || vdim <= 0 ||
         vdim % 16 || page_size <= 0 || page_size % 8)
         return 0;
-    if (ceil_div(kv * (vdim / 16), 4) > 16) return 0;
+    if (ceil_div(kv * (vdim / 16), MXM_NW) > 8) return 0;
     int rp = 1;
     while (rp < heads / kv) rp <<= 1;
     return mxm_lds_bytes(mxm_steps(dim), heads, kv, vdim, 16 / rp) <= 160 * 1024 ? 1 : 0;
@@ -409,17 +450,17 @@ extern "C" int somi_mixed_attention_mfma(const void* q, const void* k_cache, con
         hipError_t err = hipFuncSetAttribute((const void*)mixed_attention_mfma_kernel<STEPS, ACC>,                      \
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
         if (err != hipSuccess) return somi_fail("mixed_attention_mfma: %s", hipGetErrorString(err));                    \
-        hipLaunchKernelGGL((mixed_attention_mfma_kernel<STEPS, ACC>), GRID, dim3(256), lds, stream, (const bf16*)q,     \
+        hipLaunchKernelGGL((mixed_attention_mfma_kernel<STEPS, ACC>), GRID, dim3(MXM_NT), lds, stream, (const bf16*)q,  \
                            (const bf16*)k_cache, (const bf16*)v_cache, block_table, max_blocks, token_entry, positions, \
                            n_tokens, heads, kv, dim, vdim, page_size, window, scale, cap, extra, talk, v_freq,          \
                            v_pairing, rp, tq, MODE, stats, part, (bf16*)out);                                           \
     } while (0)
 #define MXM_BY_ACC(STEPS, MODE, GRID)                            \
     do {                                                         \
-        if (accs == 2) MXM_LAUNCH(STEPS, 2, MODE, GRID);         \
+        if (accs == 1) MXM_LAUNCH(STEPS, 1, MODE, GRID);         \
+        else if (accs == 2) MXM_LAUNCH(STEPS, 2, MODE, GRID);    \
         else if (accs == 4) MXM_LAUNCH(STEPS, 4, MODE, GRID);    \
-        else if (accs == 8) MXM_LAUNCH(STEPS, 8, MODE, GRID);    \
-        else MXM_LAUNCH(STEPS, 16, MODE, GRID);                  \
+        else MXM_LAUNCH(STEPS, 8, MODE, GRID);                   \
     } while (0)
 #define MXM_BY_STEPS(MODE, GRID)                         \
     do {                                                 \
