@@ -189,13 +189,13 @@ def gizilorn_config_dict(sizes: str) -> dict:
 
     def latent(kv_from=None):
         mixer = {"heads": l_heads, "dim": l_dim, "rot_dim": rot, "vdim": vdim, "kv_rank": rank, "scale": (l_dim + rot) ** -0.5,
-                 "mask": {"size": l_window}, "rot": {"base": 250000.0, "dims": rot}}
+                 "mask": {"size": l_window}, "rot": {"base": 100000.0, "dims": rot}}
         if kv_from is not None:
             mixer["kv_from"] = kv_from
         return {"type": "latent_attention", "mixer": mixer, "mlp": dense}
     attention = {"type": "attention", "mlp": dense,
                  "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "softcap": 30.0,
-                           "mask": {"size": window}, "rot": {"base": 20000.0, "dims": dim}}}
+                           "mask": {"size": window}, "rot": {"base": 10000.0, "dims": dim}}}
     return {"architecture": "Gizilorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "streams": streams,
             "layers": [latent(), latent(0), attention, attention, latent(), attention]}
 
@@ -223,7 +223,7 @@ def gizilorn_closest_attention_config_dict(sizes: str) -> dict:
     (width, streams, heads, kv_heads, dim, window, l_heads, l_dim, rot, vdim, rank, l_window, ff, vocab) = GIZILORN_SIZES[sizes]
     return {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "vocab_size": vocab, "hidden_size": width,
             "intermediate_size": ff, "num_hidden_layers": GIZILORN_LAYERS, "num_attention_heads": heads,
-            "num_key_value_heads": kv_heads, "head_dim": dim, "rope_theta": 2e4, "rms_norm_eps": 1e-6,
+            "num_key_value_heads": kv_heads, "head_dim": dim, "rope_theta": 1e4, "rms_norm_eps": 1e-6,
             "tie_word_embeddings": False, "max_position_embeddings": 32768, "hidden_act": "silu", "attention_bias": True,
             "use_sliding_window": True, "sliding_window": window, "max_window_layers": 0}
 

@@ -105,6 +105,11 @@ class ModelConfig:
     def to_dict(self) -> dict[str, Any]:
         raise NotImplementedError
 
+    def fitted_to(self, shapes: dict[str, tuple[int, ...]]) -> "ModelConfig":
+        """The configuration for a checkpoint that holds tensors of these names and shapes: an architecture whose
+        config.json may leave a size to the tensors returns a copy with that size filled in.  Default: itself."""
+        return self
+
 
 def read_config_json(model_dir: str | os.PathLike) -> dict[str, Any]:
     """Parse ``<model_dir>/config.json``; errors name the file."""

@@ -1,11 +1,11 @@
 """Typed configuration of the Gizilorn decoder: pre-norm layers around several residual streams (hyper-connections),
-whose mixer is grouped-query attention with mixed heads (capped scores, a window, one added to the softmax's
-denominator, values turned by their position) or attention over a shared low-rank latent (a window, a sigmoid gate on
+whose mixer is grouped-query attention with mixed heads (capped scores, a window, a softmax whose denominator
+holds an extra 1, values turned by their position) or attention over a shared low-rank latent (a window, a sigmoid gate on
 the heads' outputs, optionally reading the latent an earlier layer kept), with a dense feed-forward whose activation
 has two learned numbers; the embedded rows are RMS-normed.
 
-config.json keys: ``architecture`` ("Gizilorn"), ``vocab``, ``width``, ``norm.eps``, ``streams`` (absent or 1 with no
-``hc*`` tensors: the plain residual sum) and ``layers``, a list with one object per layer: ``type`` ("attention" or
+config.json keys: ``architecture`` ("Gizilorn"), ``vocab``, ``width``, ``norm.eps``, ``streams`` (absent, with no
+``hc*`` tensors in the checkpoint: the plain residual sum) and ``layers``, a list with one object per layer: ``type`` ("attention" or
 "latent_attention"), ``mixer`` with that mixer's sizes, and ``mlp`` (``{"kind": "dense", "ff": ...}`` or null).
 
 ``mixer`` of attention: ``heads``, ``kv_heads``, ``dim``, ``vdim``, ``scale``, ``softcap`` (absent: scores are not
@@ -172,6 +172,19 @@ class GizilornConfig(ModelConfig):
                 raise ConfigError(f"{where}:mixer: layer {source} keeps no latent of its own to read ('kv_from' of 'kv_from')")
             if lender.kept() != layer.mixer.kept():
                 raise ConfigError(f"{where}:mixer: 'kv_rank', 'rot_dim' and 'rot' must equal those of layer {source}, whose latent it reads")
+
+    def fitted_to(self, shapes: dict[str, tuple[int, ...]]) -> "GizilornConfig":
+        """Whether the layers have connection tensors is what the checkpoint says where config.json says one stream or
+        nothing: one stream without such tensors is the plain residual sum, and tensors of one stream without the key
+        are connections of one stream."""
+        import dataclasses
+        has = any(".hc1." in name for name in shapes)
+        if self.streams == 1 and not has:
+            return dataclasses.replace(self, streams=None)
+        if self.streams is None and has:
+            count = next(shape[0] for name, shape in shapes.items() if name.endswith(".hc1.in"))
+            return dataclasses.replace(self, streams=int(count))
+        return self
 
     @classmethod
     def from_dict(cls, data: dict[str, Any]) -> "GizilornConfig":

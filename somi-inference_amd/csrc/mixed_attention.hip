@@ -1,7 +1,7 @@
 // Grouped-query attention whose heads' softmax weights are mixed by a matrix before they meet the values.
 //
 //     s_g(i, j) = cap * tanh(scale * q_g(i) . k_kv(g)(j) / cap)            (cap = 0: scale * q . k as it is)
-//     p_g(i, j) = exp(s_g(i, j)) / (extra + sum_j' exp(s_g(i, j')))         (extra = 1: a sink with score 0 and no value)
+//     p_g(i, j) = exp(s_g(i, j)) / (extra + sum_j' exp(s_g(i, j')))         (extra = 1: as if one more key of score 0 and value 0 were seen)
 //     w_h(i, j) = sum_g T[h, g] p_g(i, j)
 //     o_h(i)    = sum_j w_h(i, j) v_kv(h)(j)
 //

@@ -1,5 +1,5 @@
 """The Gizilorn decoder as a plan: pre-norm layers around several residual streams (hyper-connections); the mixer is
-grouped-query attention with mixed heads (capped scores, a window, one added to the softmax's denominator, values
+grouped-query attention with mixed heads (capped scores, a window, a softmax whose denominator holds an extra 1, values
 rotated by their position) or attention over a shared low-rank latent (a window, a sigmoid gate on the heads' outputs;
 a layer may read the latent an earlier layer kept); a dense feed-forward whose activation has two stored numbers;
 RMS-normed embedded rows and an untied head.

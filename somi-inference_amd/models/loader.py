@@ -39,8 +39,10 @@ def load_model(model_dir: str | os.PathLike, dtype: object = "bfloat16",
                device: str | torch.device = "cuda:0") -> tuple[DecoderModel, ModelConfig]:
     """Build the model that ``<model_dir>/config.json`` names and load ``model.safetensors``."""
     arch, config = config_from_dict(read_config_json(model_dir))
+    source = SafetensorsSource(os.fspath(model_dir))
+    config = config.fitted_to({name: source.shape(name) for name in source.names()})
     model = DecoderModel(arch.build_plan(config), make_runtime(dtype, device))
-    model.load(SafetensorsSource(os.fspath(model_dir)))
+    model.load(source)
     return model, config
 
 

@@ -4,7 +4,7 @@ With H query heads over G key/value heads (query head h reads key/value head ``h
 channels and ``value_dim`` value channels a head:
 
     s_g(i, j) = scale * q_g(i) . k(j),   then, with a cap c,  s <- c * tanh(s / c)
-    p_g(i, j) = exp(s_g(i, j)) / (extra + sum_j' exp(s_g(i, j')))        extra = 1: a sink of score 0 without a value
+    p_g(i, j) = exp(s_g(i, j)) / (extra + sum_j' exp(s_g(i, j')))        extra = 1: as if one more key of score 0 and value 0 were seen
     w_h(i, j) = sum_g T[h, g] p_g(i, j)                                  T: the ``talk`` matrix [H, H]
     o_h(i)    = sum_j w_h(i, j) v(j)                                     v of head h's own key/value head
 

@@ -83,3 +83,14 @@ def test_a_lender_keeps_rows_for_its_farthest_seeing_reader():
     del data["layers"][3]["mixer"]["mask"]                   # a reader that sees everything: rows are kept for ever
     model = DecoderModel(gizilorn_plan(GizilornConfig.from_dict(data)), Runtime(torch.float32, torch.device("cpu")))
     assert model.cache_needs()[0].window is None
+
+
+def test_connection_tensors_are_what_the_checkpoint_says_for_one_stream():
+    one = GIZILORN["B"]["config"]                       # streams = 1
+    assert one.fitted_to({"l0.hc1.in": (1,), "l0.mix.q": (48, 64)}) is one
+    assert one.fitted_to({"l0.mix.q": (48, 64)}).streams is None
+    none = GIZILORN["C"]["config"]                      # no key
+    assert none.fitted_to({"l0.mix.q": (16, 80)}) is none
+    assert none.fitted_to({"l0.hc1.in": (2,), "l0.hc1.mix": (2, 2)}).streams == 2
+    three = GIZILORN["A"]["config"]
+    assert three.fitted_to({"l0.mix.q": (1, 1)}) is three          # three streams need their tensors: the loader says so

@@ -262,7 +262,7 @@ def test_the_one_in_the_denominator_and_the_mix_each_matter(dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding_of_rotated_values_far_from_the_start(dtype):
     """Values turned by positions in the hundreds and turned back by the query's: single tokens after a long prompt."""
-    part, m = mixed_part(4, 2, 16, 32, 24, 20.0, 8, base=50.0)
+    part, m = mixed_part(4, 2, 16, 32, 24, 25.0, 8, base=50.0)
     w = mixed_weights(part, 77)
     load_part(part, w, dtype, DEV)
     x = rounded(torch.randn(700, 48, generator=torch.Generator().manual_seed(9)), dtype)
@@ -393,7 +393,7 @@ def test_which_sizes_take_the_matrix_core_kernels():
 
 
 @pytest.mark.parametrize("portions", [False, True])
-@pytest.mark.parametrize("heads,kv,dim,vdim,window,cap", [(8, 4, 64, 64, 21, 20.0), (6, 2, 24, 32, None, None),
+@pytest.mark.parametrize("heads,kv,dim,vdim,window,cap", [(8, 2, 64, 32, 21, 15.0), (6, 2, 24, 32, None, None),
                                                           (5, 5, 128, 16, 100, 7.0), (16, 1, 32, 48, 3, None)])
 def test_matrix_core_and_plain_attention_agree(portions, heads, kv, dim, vdim, window, cap):
     """The two kernels on the same pages, block table and queries: tokens of three requests side by side, one of them

@@ -39,15 +39,15 @@ def random_config(rng: random.Random) -> GizilornConfig:
                 continue
             layers.append(latent(rng.choice([1, 2, 3, 6, 17, 20]), rng.choice([8, 12, 16, 32]), rng.choice([2, 4, 8, 16, 32]),
                                  rng.choice([8, 16, 24]), rng.choice([16, 24, 32, 48, 64, 96, 160]), window(),
-                                 base=rng.choice([10.0, 1000.0, 250000.0]), scale=rng.choice([0.1, 0.2, 0.4]), mlp=mlp()))
+                                 base=rng.choice([10.0, 1000.0, 100000.0]), scale=rng.choice([0.1, 0.2, 0.4]), mlp=mlp()))
             lenders.append(index)
         else:
             kv = rng.choice([1, 2, 3, 4])
             dim = rng.choice([8, 12, 16, 24, 32, 64])
             layers.append(attention(kv * rng.choice([1, 2, 3, 4, 6]), kv, dim, rng.choice([2, 8, 16, 24, 32, 48, 64]), window(),
-                                    rng.choice([None, 5.0, 20.0, 50.0]), rng.choice([d for d in (2, 4, 8, 12, 16, 32, 64) if d <= dim]),
-                                    base=rng.choice([10.0, 1000.0, 20000.0]), scale=rng.choice([0.1, 0.2, 0.4]), mlp=mlp()))
-    return GizilornConfig(vocab=rng.choice([61, 97, 130, 256, 301]), width=rng.choice([40, 44, 64, 72, 100, 136]),
+                                    rng.choice([None, 5.0, 25.0, 50.0]), rng.choice([d for d in (2, 4, 8, 12, 16, 32, 64) if d <= dim]),
+                                    base=rng.choice([10.0, 1000.0, 50000.0]), scale=rng.choice([0.1, 0.2, 0.4]), mlp=mlp()))
+    return GizilornConfig(vocab=rng.choice([61, 97, 130, 256, 301]), width=rng.choice([40, 44, 64, 72, 100, 132]),
                           norm_eps=rng.choice([1e-6, 1e-5]), streams=rng.choice([None, 1, 2, 3, 4, 8]), layers=tuple(layers))
 
 
